@@ -1,0 +1,143 @@
+/*
+ * pilotann.h — C ABI of the MI355X search stage of PilotANN.
+ *
+ * Plain pointers and sizes only; every device pointer is memory of the GPU
+ * that is current when the call is made, every call enqueues on the HIP
+ * stream it is given (hipStream_t passed as void*, NULL = the null stream)
+ * and returns without synchronising unless it says otherwise.
+ *
+ * Return value: 0 on success; < 0 an argument error (PA_E_*), detected on the
+ * host before anything is launched; > 0 a hipError_t from the runtime.
+ * pa_error_string() turns either into text.
+ *
+ * Each entry point names the reference interface it replaces (paths under
+ * the reference repository).
+ */
+#ifndef PILOTANN_H
+#define PILOTANN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PA_BEAM_WIDTH 4     /* traverse_cuda.cu:13  — output is [B, 4, ef]      */
+#define PA_MAX_NEIGHBORS 64 /* traverse_cuda.cu:280 — 4 * n_neighbors <= 256    */
+#define PA_MAX_EF_TOTAL 2048 /* traverse_cpu.cpp:250 — largest heap of the ladder */
+
+enum {
+    PA_OK = 0,
+    PA_E_NULL = -1,        /* a required pointer is NULL                         */
+    PA_E_SHAPE = -2,       /* a size is negative or inconsistent                 */
+    PA_E_DIM = -3,         /* vector length not a multiple of 8 (distance.h:35-36) */
+    PA_E_NEIGHBORS = -4,   /* n_neighbors outside 1..64                          */
+    PA_E_EF = -5,          /* beam * ef outside 1..2048                          */
+    PA_E_WORKSPACE = -6,   /* workspace smaller than pa_traverse_plan() asked    */
+    PA_E_GRAPH = -7,       /* pa_graph_prepare found a malformed graph           */
+    PA_E_LEAVES = -8,      /* n_leaves not a multiple of 32 (routing_cuda.cu:90) */
+    PA_E_CHUNK = -9,       /* batch not a multiple of chunk (pipeline_cpu.cpp:58) */
+    PA_E_RANGE = -10       /* an id does not fit 31 bits                         */
+};
+
+const char *pa_error_string(int code);
+
+/* Heap size the host search uses for a given ef_search
+ * (traverse_cpu.cpp:228-254): 16,32,48,64,96,128,192,256,384,512,1024,2048;
+ * -1 above 2048. */
+int pa_heap_size(int ef_search);
+
+/* ---- device graph -------------------------------------------------------- */
+
+/*
+ * Builds the device-resident form of a subgraph once per index
+ * (the reference re-reads indptr / indices / mapping as int64 on every
+ * expansion: traverse_cuda.cu:130-140,199).
+ *
+ *   indptr  [n_nodes + 1], indices [indptr[n_nodes]], mapping [n_nodes]:
+ *           the int64 device arrays `traverse_cuda` receives
+ *           (traverse_cuda.cu:249-258); indices are global ids, mapping is
+ *           global id -> row of `storage` or -1.
+ *   adj     [n_storage * n_neighbors] int32, out: row r lists, in order, the
+ *           storage rows of the neighbours of the node stored in row r, cut
+ *           at the first negative id (traverse_cpu.cpp:107-109), without
+ *           self loops, repeats of an earlier entry of the same row, or
+ *           neighbours that have no storage row; -1 pads.  Dropping those
+ *           entries does not change what a search does: each of them is
+ *           already marked visited when the row is scanned.
+ *   gid     [n_storage] int32, out: storage row -> global id.
+ *   status  [1] int32 device word, out: 0, or a bit set: 1 = mapping is not
+ *           a bijection onto 0..n_storage-1, 2 = a row is longer than
+ *           n_neighbors, 4 = an id is >= n_nodes.
+ *
+ * Synchronises the stream and returns PA_E_GRAPH when status != 0.
+ */
+int pa_graph_prepare(const int64_t *indptr, const int64_t *indices,
+                     const int64_t *mapping, int64_t n_nodes,
+                     int64_t n_storage, int n_neighbors, int32_t *adj,
+                     int32_t *gid, int32_t *status, void *stream);
+
+/* ---- traversal ----------------------------------------------------------- */
+
+/*
+ * Sizes the scratch memory pa_traverse needs: one visited bitmask of
+ * n_storage bits per resident wavefront plus a work counter.  n_slots
+ * (out, may be NULL) is the number of wavefronts that will be launched.
+ */
+int pa_traverse_plan(int64_t n_storage, int64_t batch, int dp, int ef_total,
+                     int *n_slots, size_t *workspace_bytes);
+
+/*
+ * Replaces `traverse_cuda` (extension/traverse_cuda.cu:249-316,
+ * pilot_ann/kernels/__init__.py:62-75).
+ *
+ * Per query: the best-first search of the host kernel
+ * (extension/traverse_cpu.cpp:12-163) with ef_search = k = beam * ef on the
+ * prepared subgraph, distances over the dp stored coordinates.  One
+ * wavefront runs one query.
+ *
+ *   out_I [batch * beam * ef] int64, out_D [same] float: the k results of
+ *         query b start at b * k, best first; unused slots hold -1 / +inf
+ *         at the end.  Ids are global.
+ *   adj, gid: from pa_graph_prepare.   mapping [n_nodes] int64 as there.
+ *   storage [n_storage * dp] float, query [batch * dp] float.
+ *   init_I / init_D [batch * n_init]: entry ids (global, negative = unused)
+ *         and their squared distances over the same dp coordinates.
+ *   counters: NULL, or 5 uint64 device words that are incremented by
+ *         {nodes expanded, adjacency entries read, distances evaluated,
+ *          candidates admitted, result slots written}.
+ *   workspace: at least pa_traverse_plan()'s bytes, 256-byte aligned, not
+ *         shared with a call that may run at the same time.
+ */
+int pa_traverse(int64_t *out_I, float *out_D, const int32_t *adj,
+                const int32_t *gid, const int64_t *mapping,
+                const float *storage, const float *query,
+                const int64_t *init_I, const float *init_D, int64_t batch,
+                int64_t n_nodes, int64_t n_storage, int dp, int n_init,
+                int beam, int ef, int n_neighbors, void *workspace,
+                size_t workspace_bytes, uint64_t *counters, void *stream);
+
+/* ---- entry router -------------------------------------------------------- */
+
+/*
+ * Replaces `routing_cuda` (extension/routing_cuda.cu:70-113,
+ * pilot_ann/kernels/__init__.py:97-103).
+ *
+ *   router [batch] int64, out: index of the nearest route vector.
+ *   dist   [batch * n_leaves] float, out: squared L2 from the query to each
+ *          leaf vector of its route, entry_vectors[router[b], l, :].
+ *   query [batch * dp], route_vectors [n_routers * dp],
+ *   entry_vectors [n_routers * n_leaves * dp], all float.
+ * With n_routers == 0 every query uses group 0 of entry_vectors and `router`
+ * may be NULL: the distances of a fixed entry list
+ * (pilot_ann/layers/entry.py:70-77).
+ */
+int pa_route(int64_t *router, float *dist, const float *query,
+             const float *route_vectors, const float *entry_vectors,
+             int64_t batch, int n_routers, int n_leaves, int dp, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PILOTANN_H */

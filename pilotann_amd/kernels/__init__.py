@@ -1,0 +1,258 @@
+"""Operator API with the call signatures of ``pilot_ann/kernels/__init__.py``.
+
+Every function validates its tensors the way the reference's ``CHECK_CPU`` /
+``CHECK_CUDA`` macros do (``extension/inc/common.h:15-29``: device, rank,
+dtype, contiguity; ``RuntimeError`` on violation) and then calls the C ABI of
+``csrc/libpilotann.so``.  Device work is enqueued on torch's current stream
+and not synchronised, like the reference (``traverse_cuda.cu:284``,
+``routing_cuda.cu:103``).
+"""
+import ctypes
+from collections import OrderedDict
+
+import torch
+
+from .. import _lib
+
+BEAM_WIDTH = 4
+
+
+# ---- argument checks --------------------------------------------------------
+
+def _check(x, name, dim, dtype, cuda):
+    if not isinstance(x, torch.Tensor):
+        raise RuntimeError(f'{name} must be a tensor')
+    if cuda and not x.is_cuda:
+        raise RuntimeError(f'{name} must be a CUDA tensor')
+    if not cuda and x.is_cuda:
+        raise RuntimeError(f'{name} must be a CPU tensor')
+    if x.dim() != dim:
+        raise RuntimeError(f'{name} must be of dim {dim}')
+    if x.dtype != dtype:
+        raise RuntimeError(f'{name} must be type of {dtype}')
+    if not x.is_contiguous():
+        raise RuntimeError(f'{name} custom kernel requires contiguous tensor')
+
+
+def _require(cond, text):
+    if not cond:
+        raise RuntimeError(f'Expected {text} to be true, but got false.')
+
+
+def _ptr(x):
+    return ctypes.c_void_p(x.data_ptr() if x is not None else None)
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+# ---- device graph -----------------------------------------------------------
+
+class PreparedGraph:
+    """Device-resident search form of a subgraph (see ``pa_graph_prepare``):
+    ``adj[n_storage, n_neighbors]`` int32 storage rows, ``gid[n_storage]``
+    int32 global ids, plus the int64 ``mapping`` the caller supplied."""
+
+    def __init__(self, indptr, indices, mapping, n_storage, n_neighbors):
+        _check(indptr, 'indptr', 1, torch.int64, True)
+        _check(indices, 'indices', 1, torch.int64, True)
+        _check(mapping, 'mapping', 1, torch.int64, True)
+        n_nodes = indptr.size(0) - 1
+        _require(mapping.size(0) == n_nodes, 'mapping.size(0) == n_nodes')
+        self.n_nodes = n_nodes
+        self.n_storage = int(n_storage)
+        self.n_neighbors = int(n_neighbors)
+        self.mapping = mapping
+        self._sources = (indptr, indices)
+        dev = indptr.device
+        self.adj = torch.empty(self.n_storage * self.n_neighbors,
+                               dtype=torch.int32, device=dev)
+        self.gid = torch.empty(self.n_storage, dtype=torch.int32, device=dev)
+        self.status = torch.zeros(1, dtype=torch.int32, device=dev)
+        with torch.cuda.device(dev):
+            rc = _lib.lib().pa_graph_prepare(
+                _ptr(indptr), _ptr(indices), _ptr(mapping), n_nodes,
+                self.n_storage, self.n_neighbors, _ptr(self.adj),
+                _ptr(self.gid), _ptr(self.status), _stream())
+        if rc == -7:
+            raise RuntimeError(
+                'pa_graph_prepare: malformed graph, status bits '
+                f'{int(self.status.item())} (1 mapping not a bijection, '
+                '2 row longer than n_neighbors, 4 id out of range)')
+        _lib.check(rc, 'pa_graph_prepare')
+
+
+_graph_cache = OrderedDict()
+_GRAPH_CACHE_SIZE = 4
+
+
+def prepare_graph(indptr, indices, mapping, n_storage, n_neighbors):
+    """Cached :class:`PreparedGraph` for these three tensors.  The cache holds
+    the tensors themselves, so an address cannot come back with other
+    content; an in-place change bumps the tensor's version and misses."""
+    key = (indptr.data_ptr(), indices.data_ptr(), mapping.data_ptr(),
+           indptr._version, indices._version, mapping._version,
+           indptr.numel(), indices.numel(), int(n_storage), int(n_neighbors),
+           str(indptr.device))
+    hit = _graph_cache.get(key)
+    if hit is not None:
+        _graph_cache.move_to_end(key)
+        return hit
+    graph = PreparedGraph(indptr, indices, mapping, n_storage, n_neighbors)
+    _graph_cache[key] = graph
+    while len(_graph_cache) > _GRAPH_CACHE_SIZE:
+        _graph_cache.popitem(last=False)
+    return graph
+
+
+_workspaces = {}
+
+
+def _workspace(device, nbytes):
+    """Scratch memory for one traversal call, one buffer per (device,
+    stream): calls on different streams may overlap and must not share it."""
+    key = (str(device), torch.cuda.current_stream(device).cuda_stream)
+    buf = _workspaces.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8,
+                          device=device)
+        _workspaces[key] = buf
+    return buf
+
+
+# ---- traversal --------------------------------------------------------------
+
+def traverse_cuda(output_I: torch.Tensor,
+                  output_D: torch.Tensor,
+                  indptr: torch.Tensor,
+                  indices: torch.Tensor,
+                  mapping: torch.Tensor,
+                  storage: torch.Tensor,
+                  query: torch.Tensor,
+                  initial_I: torch.Tensor,
+                  initial_D: torch.Tensor,
+                  n_neighbors: int,
+                  counters: torch.Tensor = None):
+    """Same arguments as ``kernels.traverse_cuda``
+    (``pilot_ann/kernels/__init__.py:62-75``; checks of
+    ``traverse_cuda.cu:256-281``).  ``output_*`` are ``[B, 4, ef]``; row b,
+    flattened, receives the ``4·ef`` best candidates of the host search
+    (``traverse_cpu.cpp:12-163`` with ``ef_search = k = 4·ef``) best first,
+    ``-1`` / ``+inf`` in unused slots.  ``n_neighbors`` may be any value up
+    to 64.  ``counters`` (5 int64 on the device) is an optional work tally.
+    """
+    _check(indptr, 'indptr', 1, torch.int64, True)
+    _check(indices, 'indices', 1, torch.int64, True)
+    _check(mapping, 'mapping', 1, torch.int64, True)
+    _check(storage, 'storage', 2, torch.float32, True)
+    _check(query, 'query', 2, torch.float32, True)
+    _check(initial_I, 'initial_I', 2, torch.int64, True)
+    _check(initial_D, 'initial_D', 2, torch.float32, True)
+    _check(output_I, 'output_I', 3, torch.int64, True)
+    _check(output_D, 'output_D', 3, torch.float32, True)
+    d_model = query.size(-1)
+    batch_size = query.size(0)
+    n_nodes = indptr.size(0) - 1
+    n_storage = storage.size(0)
+    ef_search = output_I.size(-1)
+    _require(mapping.size(0) == n_nodes, 'mapping.size(0) == n_nodes')
+    _require(storage.size(-1) == d_model, 'storage.size(-1) == d_model')
+    _require(output_I.size(0) == batch_size, 'output_I.size(0) == batch_size')
+    _require(output_I.size(1) == BEAM_WIDTH, 'output_I.size(1) == BEAM_WIDTH')
+    _require(initial_I.size(0) == batch_size,
+             'initial_I.size(0) == batch_size')
+    _require(output_I.size() == output_D.size(),
+             'output_I.sizes() == output_D.sizes()')
+    _require(initial_I.size() == initial_D.size(),
+             'initial_I.sizes() == initial_D.sizes()')
+    _require(1 <= n_neighbors <= 64, '1 <= n_neighbors <= 64')
+    _require(BEAM_WIDTH * ef_search <= 2048, 'heapq_size supported')
+    _require(d_model % 8 == 0, 'd_model % 8 == 0')
+    if counters is not None:
+        _check(counters, 'counters', 1, torch.int64, True)
+        _require(counters.numel() >= 5, 'counters.numel() >= 5')
+
+    graph = prepare_graph(indptr, indices, mapping, n_storage, n_neighbors)
+    traverse_prepared(output_I, output_D, graph, storage, query, initial_I,
+                      initial_D, counters)
+
+
+def traverse_prepared(output_I, output_D, graph: PreparedGraph, storage,
+                      query, initial_I, initial_D, counters=None):
+    """:func:`traverse_cuda` on an already prepared graph (no checks beyond
+    the C ABI's own)."""
+    lib = _lib.lib()
+    batch_size, d_model = query.shape
+    ef_search = output_I.size(-1)
+    beam = output_I.size(1)
+    with torch.cuda.device(query.device):
+        nbytes = ctypes.c_size_t()
+        _lib.check(lib.pa_traverse_plan(
+            graph.n_storage, batch_size, d_model, beam * ef_search, None,
+            ctypes.byref(nbytes)), 'pa_traverse_plan')
+        ws = _workspace(query.device, nbytes.value)
+        _lib.check(lib.pa_traverse(
+            _ptr(output_I), _ptr(output_D), _ptr(graph.adj), _ptr(graph.gid),
+            _ptr(graph.mapping), _ptr(storage), _ptr(query), _ptr(initial_I),
+            _ptr(initial_D), batch_size, graph.n_nodes, graph.n_storage,
+            d_model, initial_I.size(-1), beam, ef_search, graph.n_neighbors,
+            _ptr(ws), ws.numel(), _ptr(counters), _stream()), 'pa_traverse')
+
+
+# ---- entry router -----------------------------------------------------------
+
+def routing_cuda(query: torch.Tensor,
+                 route_vectors: torch.Tensor,
+                 entry_nodes: torch.Tensor,
+                 entry_vectors: torch.Tensor):
+    """``kernels.routing_cuda`` (``pilot_ann/kernels/__init__.py:97-103``,
+    checks of ``routing_cuda.cu:76-90``): returns ``(router[B] int64,
+    distances[B, n_leaves] float32)``."""
+    _check(query, 'query', 2, torch.float32, True)
+    _check(route_vectors, 'route_vectors', 2, torch.float32, True)
+    _check(entry_vectors, 'entry_vectors', 3, torch.float32, True)
+    _check(entry_nodes, 'entry_nodes', 2, torch.int64, True)
+    d_model = query.size(-1)
+    batch_size = query.size(0)
+    n_leaves = entry_nodes.size(-1)
+    n_routers = route_vectors.size(0)
+    _require(route_vectors.size(-1) == d_model,
+             'route_vectors.size(-1) == d_model')
+    _require(entry_vectors.size(-1) == d_model,
+             'entry_vectors.size(-1) == d_model')
+    _require(entry_vectors.size(0) == n_routers,
+             'entry_vectors.size(0) == n_routers')
+    _require(entry_vectors.size(1) == n_leaves,
+             'entry_vectors.size(1) == n_leaves')
+    _require(n_leaves % 32 == 0, 'n_leaves % BLOCK_SIZE == 0')
+    _require(d_model % 8 == 0, 'd_model % 8 == 0')
+    router = torch.empty(batch_size, dtype=torch.int64, device=query.device)
+    distances = torch.empty(batch_size, n_leaves, dtype=torch.float32,
+                            device=query.device)
+    with torch.cuda.device(query.device):
+        _lib.check(_lib.lib().pa_route(
+            _ptr(router), _ptr(distances), _ptr(query), _ptr(route_vectors),
+            _ptr(entry_vectors), batch_size, n_routers, n_leaves, d_model,
+            _stream()), 'pa_route')
+    return router, distances
+
+
+def entry_distances(query: torch.Tensor, entry_vectors: torch.Tensor):
+    """Squared L2 from every query to a fixed list of entry vectors
+    ``[n_entries, d]`` — what ``IndexEntry.search`` computes with
+    ``cdist().square()`` in its random mode (``layers/entry.py:70-74``),
+    here with the traversal's own distance kernel."""
+    _check(query, 'query', 2, torch.float32, True)
+    _check(entry_vectors, 'entry_vectors', 2, torch.float32, True)
+    _require(entry_vectors.size(-1) == query.size(-1),
+             'entry_vectors.size(-1) == d_model')
+    _require(query.size(-1) % 8 == 0, 'd_model % 8 == 0')
+    distances = torch.empty(query.size(0), entry_vectors.size(0),
+                            dtype=torch.float32, device=query.device)
+    with torch.cuda.device(query.device):
+        _lib.check(_lib.lib().pa_route(
+            None, _ptr(distances), _ptr(query), None, _ptr(entry_vectors),
+            query.size(0), 0, entry_vectors.size(0), query.size(-1),
+            _stream()), 'pa_route')
+    return distances

@@ -1,0 +1,37 @@
+"""Seeded synthetic data in the shapes the benchmark configurations name."""
+import torch
+
+
+def gaussian_mixture(n: int, d: int, n_centers: int, sigma: float, seed: int,
+                     normalize: bool = False, device: str = 'cpu',
+                     center_seed: int = None):
+    """``n`` points of an isotropic Gaussian mixture: centres ~ N(0, I_d),
+    a uniformly drawn centre plus ``sigma``·N(0, I_d) per point; optionally
+    projected onto the unit sphere.  ``center_seed`` fixes the centres apart
+    from the points, so that queries (another ``seed``) share the base set's
+    mixture."""
+    gc = torch.Generator(device='cpu').manual_seed(
+        seed if center_seed is None else center_seed)
+    centers = torch.randn(n_centers, d, generator=gc)
+    g = torch.Generator(device='cpu').manual_seed(seed + 7919)
+    which = torch.randint(high=n_centers, size=[n], generator=g)
+    out = torch.empty(n, d, device=device)
+    centers = centers.to(device)
+    for lo in range(0, n, 131072):
+        hi = min(n, lo + 131072)
+        noise = torch.randn(hi - lo, d, generator=g).to(device)
+        out[lo:hi] = centers[which[lo:hi].to(device)] + sigma * noise
+    if normalize:
+        out = torch.nn.functional.normalize(out, dim=-1)
+    return out
+
+
+def brute_force_topk(query: torch.Tensor, storage: torch.Tensor, k: int,
+                     chunk: int = 1024):
+    """Exact k nearest rows of ``storage`` (squared L2) for every query."""
+    norms = storage.square().sum(-1)
+    ids = []
+    for q in torch.split(query, chunk):
+        d = norms.unsqueeze(0) - 2.0 * (q @ storage.T)
+        ids.append(torch.topk(d, k=k, dim=-1, largest=False).indices)
+    return torch.cat(ids)

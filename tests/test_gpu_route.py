@@ -1,0 +1,69 @@
+"""Router against the oracle: route ids equal to the exact argmin except on
+float ties, leaf distances bit-identical."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from pilotann_amd import kernels, utils
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize('R,L,d,B', [(8, 32, 64, 1), (16, 64, 200, 777),
+                                     (32, 32, 64, 1023), (64, 64, 128, 2500),
+                                     (40, 96, 32, 333)])
+def test_routing_matches_oracle(R, L, d, B, device):
+    x = utils.gaussian_mixture(20000, d, 32, 0.5, seed=R + L)
+    q = utils.gaussian_mixture(B, d, 32, 0.5, seed=99, center_seed=R + L)
+    route_vectors, entry_nodes = utils.router_init(x, None, R, L, seed=1)
+    entry_vectors = x[entry_nodes].contiguous()
+    router, dist = kernels.routing_cuda(
+        q.to(device), route_vectors.contiguous().to(device),
+        entry_nodes.to(device), entry_vectors.to(device))
+    router, dist = router.cpu().numpy(), dist.cpu().numpy()
+    ref_router, _ = oracle.route(q.numpy(), route_vectors.contiguous().numpy(),
+                                 entry_vectors.numpy())
+    # the chosen route is the nearest one up to float rounding
+    exact = torch.cdist(q.double(), route_vectors.double()).square().numpy()
+    chosen = exact[np.arange(B), router]
+    assert (chosen <= exact.min(-1) * (1 + 1e-5) + 1e-6).all()
+    assert (router == ref_router).mean() > 0.999
+    # distances to the leaves of the chosen route: bit-identical
+    ref = np.stack([
+        oracle.square_dist(q[b].numpy(), x.numpy(),
+                           entry_nodes[router[b]].numpy().copy())
+        for b in range(B)])
+    assert np.array_equal(dist, ref)
+    # the reference's own check (test_routing.py:69-85)
+    target = torch.cdist(q.unsqueeze(1), x[entry_nodes[router]]).square()
+    assert torch.allclose(torch.from_numpy(dist), target.squeeze(1), atol=1e-3)
+
+
+def test_entry_distances(device):
+    x = utils.gaussian_mixture(5000, 96, 8, 0.5, seed=5)
+    q = utils.gaussian_mixture(300, 96, 8, 0.5, seed=6, center_seed=5)
+    nodes = torch.randint(high=5000, size=[48],
+                          generator=torch.Generator().manual_seed(0))
+    dist = kernels.entry_distances(q.to(device), x[nodes].contiguous().to(device))
+    ref = np.stack([oracle.square_dist(q[b].numpy(), x.numpy(),
+                                       nodes.numpy().copy())
+                    for b in range(300)])
+    assert np.array_equal(dist.cpu().numpy(), ref)
+
+
+def test_routing_argument_errors(device):
+    q = torch.randn(4, 64, device=device)
+    rv = torch.randn(8, 64, device=device)
+    en = torch.zeros(8, 32, dtype=torch.long, device=device)
+    ev = torch.randn(8, 32, 64, device=device)
+    kernels.routing_cuda(q, rv, en, ev)
+    with pytest.raises(RuntimeError):
+        kernels.routing_cuda(q.cpu(), rv, en, ev)
+    with pytest.raises(RuntimeError):
+        kernels.routing_cuda(q, rv[:, :32], en, ev)
+    with pytest.raises(RuntimeError):
+        kernels.routing_cuda(q, rv, en[:, :24].contiguous(),
+                             ev[:, :24].contiguous())
+    with pytest.raises(RuntimeError):
+        kernels.routing_cuda(q, rv, en.int(), ev)

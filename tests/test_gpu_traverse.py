@@ -1,0 +1,137 @@
+"""GPU traversal against the CPU oracle on identical graph, entries and
+reduced vectors.  Bar: distances bit-identical, ids identical except within
+exact distance ties (tests/common.py:assert_same_search)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from pilotann_amd import kernels
+from common import Problem, assert_same_search
+
+pytestmark = pytest.mark.gpu
+
+
+def run_gpu(p, dp, ef, init_I, init_D, device, counters=False):
+    B = p.query.size(0)
+    out_I = torch.empty(B, 4, ef, dtype=torch.long, device=device)
+    out_D = torch.empty(B, 4, ef, dtype=torch.float, device=device)
+    cnt = torch.zeros(5, dtype=torch.long, device=device) if counters else None
+    storage = p.x[p.nodelist][:, :dp].contiguous().to(device)
+    kernels.traverse_cuda(
+        output_I=out_I, output_D=out_D,
+        indptr=p.sub_indptr.to(device), indices=p.sub_indices.to(device),
+        mapping=p.mapping.to(device), storage=storage,
+        query=p.query[:, :dp].contiguous().to(device),
+        initial_I=init_I.to(device), initial_D=init_D.to(device),
+        n_neighbors=p.deg, counters=cnt)
+    torch.cuda.synchronize()
+    return (out_I.flatten(1).cpu().numpy(), out_D.flatten(1).cpu().numpy(),
+            None if cnt is None else cnt.cpu().numpy())
+
+
+def run_oracle(p, dp, ef, init_I, init_D, counters=None):
+    B = p.query.size(0)
+    k = 4 * ef
+    out_I = np.empty((B, k), np.int64)
+    out_D = np.empty((B, k), np.float32)
+    oracle.traverse_cpu(
+        out_I, out_D, init_I.numpy().copy(), init_D.numpy().copy(),
+        p.sub_indptr.numpy(), p.sub_indices.numpy(),
+        np.ascontiguousarray(p.x[:, :dp].numpy()),
+        np.ascontiguousarray(p.query[:, :dp].numpy()), k, counters)
+    return out_I, out_D
+
+
+CASES = [
+    # n, d, dp, deg, graph, ratio, ef, n_init, reference-style padding
+    (4000, 32, 32, 32, 'nsw', 0.25, 16, 32, False),
+    (4000, 32, 32, 32, 'nsg', 0.25, 64, 32, True),
+    (6000, 64, 32, 32, 'nsw', 0.5, 8, 64, False),
+    (6000, 96, 64, 48, 'nsg', 0.25, 32, 32, False),
+    (8000, 128, 128, 64, 'nsw', 0.25, 64, 64, True),
+    (3000, 64, 40, 24, 'nsw', None, 24, 16, False),
+    (5000, 64, 64, 64, 'nsw', 0.5, 128, 64, False),
+    (5000, 32, 32, 32, 'nsw', 0.5, 512, 32, False),
+]
+
+
+@pytest.mark.parametrize('case', CASES, ids=[str(c) for c in CASES])
+def test_traverse_matches_oracle(case, device):
+    n, d, dp, deg, gtype, ratio, ef, n_init, pad = case
+    print('case', case, flush=True)
+    p = Problem(n=n, d=d, deg=deg, graph_type=gtype, sample_ratio=ratio,
+                seed=n + ef, n_query=96, pad_like_reference=pad)
+    init_I, init_D = p.entries(n_init, seed=5, dp=dp)
+    I_ref, D_ref = run_oracle(p, dp, ef, init_I, init_D)
+    I_gpu, D_gpu, _ = run_gpu(p, dp, ef, init_I, init_D, device)
+    assert_same_search(I_gpu, D_gpu, I_ref, D_ref)
+    # layout: best first, unused slots -1 / +inf at the end
+    finite = np.isfinite(D_gpu)
+    assert (np.diff(np.where(finite, D_gpu, np.inf), axis=1) >= 0).all()
+    assert ((I_gpu >= 0) == finite).all()
+
+
+def test_counters_match_oracle(device):
+    p = Problem(n=5000, d=64, deg=32, sample_ratio=0.25, seed=11, n_query=128)
+    init_I, init_D = p.entries(32, seed=6, dp=32, sampled_only=True)
+    ref = np.zeros(5, np.int64)
+    I_ref, D_ref = run_oracle(p, 32, 16, init_I, init_D, ref)
+    I_gpu, D_gpu, cnt = run_gpu(p, 32, 16, init_I, init_D, device, True)
+    assert_same_search(I_gpu, D_gpu, I_ref, D_ref)
+    # expansions, distance evaluations and admissions are the same events
+    assert cnt[0] == ref[0] and cnt[2] == ref[2] and cnt[3] == ref[3]
+    assert cnt[4] == 128 * 64
+
+
+def test_duplicate_and_unused_entries(device):
+    p = Problem(n=3000, d=32, deg=32, sample_ratio=0.5, seed=3, n_query=64)
+    init_I, init_D = p.entries(16, seed=7)
+    init_I[:, 3] = init_I[:, 2]
+    init_D[:, 3] = init_D[:, 2]
+    init_I[:, 5] = -1
+    I_ref, D_ref = run_oracle(p, 32, 8, init_I, init_D)
+    I_gpu, D_gpu, _ = run_gpu(p, 32, 8, init_I, init_D, device)
+    assert_same_search(I_gpu, D_gpu, I_ref, D_ref)
+
+
+def test_repeat_is_deterministic_and_reuses_workspace(device):
+    p = Problem(n=4000, d=32, deg=32, sample_ratio=0.25, seed=21, n_query=200)
+    init_I, init_D = p.entries(32, seed=8)
+    a = run_gpu(p, 32, 32, init_I, init_D, device)
+    b = run_gpu(p, 32, 32, init_I, init_D, device)
+    assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
+
+
+def test_argument_errors(device):
+    p = Problem(n=2000, d=32, deg=32, sample_ratio=0.5, seed=4, n_query=8)
+    init_I, init_D = p.entries(8, seed=1)
+    args = dict(
+        output_I=torch.empty(8, 4, 16, dtype=torch.long, device=device),
+        output_D=torch.empty(8, 4, 16, dtype=torch.float, device=device),
+        indptr=p.sub_indptr.to(device), indices=p.sub_indices.to(device),
+        mapping=p.mapping.to(device),
+        storage=p.x[p.nodelist].contiguous().to(device),
+        query=p.query.to(device), initial_I=init_I.to(device),
+        initial_D=init_D.to(device), n_neighbors=32)
+    kernels.traverse_cuda(**args)
+    for key, bad in [
+        ('query', args['query'].cpu()),
+        ('indices', args['indices'].int()),
+        ('output_I', args['output_I'][:, :2]),
+        ('output_D', torch.empty(8, 4, 8, dtype=torch.float, device=device)),
+        ('storage', args['storage'][:, :24]),
+        ('n_neighbors', 65),
+        ('initial_I', args['initial_I'][:4]),
+    ]:
+        with pytest.raises(RuntimeError):
+            kernels.traverse_cuda(**{**args, key: bad})
+    with pytest.raises(RuntimeError):
+        kernels.traverse_cuda(**{
+            **args,
+            'output_I': torch.empty(8, 4, 1024, dtype=torch.long, device=device),
+            'output_D': torch.empty(8, 4, 1024, dtype=torch.float, device=device)})
+    # a row longer than n_neighbors is a malformed graph
+    with pytest.raises(RuntimeError):
+        kernels.traverse_cuda(**{**args, 'n_neighbors': 16})
+    torch.cuda.synchronize()
