@@ -1,0 +1,287 @@
+"""Benchmark of the GPU search stage (entry router + subgraph traversal) on
+one MI355X, on seeded synthetic data in the shape of the headline
+configuration: 1M x 768 fp32 unit-norm vectors from a 1024-component mixture,
+SVD to d_principle = 128, sample_ratio 0.25, a 64-neighbour base-layer graph
+(HNSW M = 32 shape), router64x64, 10k queries, top-10.
+
+A step = one pass of the hot path over the 10k-query batch: `routing_cuda`
+then `traverse_cuda`, inputs resident in HBM, at the smallest ef of the sweep
+whose end-to-end recall@10 (after the host refine) reaches 0.90.  One JSON
+line is printed; `value` is queries per second of that step.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+                    [--n-base N] [--queries B] [--ef EF] [--no-cpu-baseline]
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+METRIC = 'QPS @ recall@10>=0.90 (1M x 768 fp32, 1 GPU); traversal HBM GB/s'
+HBM_PEAK_GBS = 8000.0
+
+CONFIGS = {
+    # BASELINE.json configs[2]: the configuration the metric is quoted on
+    'c3': dict(n=1_000_000, d=768, dp=128, n_centers=1024, sigma=1.0,
+               decay=0.5, normalize=True, ratio=0.25, graph='nsw64',
+               entry='router64x64', queries=10_000, k=10,
+               ef_sweep=[4, 8, 16, 24, 32, 48, 64], seed=301),
+    # BASELINE.json configs[1]
+    'c2': dict(n=1_000_000, d=96, dp=64, n_centers=256, sigma=1.0,
+               decay=0.5, normalize=False, ratio=0.25, graph='nsw32',
+               entry='router32x32', queries=10_000, k=10,
+               ef_sweep=[8, 16, 32, 64, 128], seed=201),
+}
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def build_index(cfg, device):
+    from pilotann_amd import IndexStaged, utils
+    t0 = time.time()
+    x = utils.gaussian_mixture(
+        cfg['n'], cfg['d'], cfg['n_centers'], cfg['sigma'], seed=cfg['seed'],
+        normalize=cfg['normalize'], device=device, decay=cfg['decay'])
+    q = utils.gaussian_mixture(
+        cfg['queries'], cfg['d'], cfg['n_centers'], cfg['sigma'],
+        seed=cfg['seed'] + 1, normalize=cfg['normalize'], device=device,
+        decay=cfg['decay'], center_seed=cfg['seed'])
+    target = utils.brute_force_topk(q, x, cfg['k']).cpu()
+    log(f'[bench] data + ground truth {time.time() - t0:.1f}s')
+    index = IndexStaged(d_model=cfg['d'], d_principle=cfg['dp'],
+                        sample_ratio=cfg['ratio'], graph_method=cfg['graph'],
+                        entry_method=cfg['entry'], seed=cfg['seed'],
+                        build_device=device)
+    index.train(x)
+    del x
+    torch.cuda.empty_cache()
+    index.to(device)
+    log(f'[bench] index built {time.time() - t0:.1f}s, '
+        f'sampled {index.nodelist.numel()} of {cfg["n"]}')
+    return index, q.cpu(), target
+
+
+class Stage:
+    """The timed hot path: router then traversal, device resident."""
+
+    def __init__(self, index, query, device):
+        from pilotann_amd import kernels
+        self.kernels = kernels
+        self.index = index
+        self.device = device
+        self.query_rot = torch.matmul(query, index.VT.T).contiguous()
+        self.query_cuda = self.query_rot[:, :index.d_principle].contiguous().to(device)
+        self.graph = kernels.prepare_graph(
+            index.subgraph_cuda.indptr, index.subgraph_cuda.indices,
+            index.mapping_cuda, index.storage_cuda.size(0), index.n_neighbors)
+        self.B = query.size(0)
+        self.out = {}
+
+    def buffers(self, ef):
+        if ef not in self.out:
+            self.out[ef] = (
+                torch.empty(self.B, 4, ef, dtype=torch.long, device=self.device),
+                torch.empty(self.B, 4, ef, dtype=torch.float, device=self.device))
+        return self.out[ef]
+
+    def entries(self):
+        EP_I, EP_D = self.index.entry.search(self.query_cuda)
+        return EP_I.contiguous(), EP_D.contiguous()
+
+    def traverse(self, ef, EP_I, EP_D, counters=None):
+        out_I, out_D = self.buffers(ef)
+        self.kernels.traverse_prepared(
+            out_I, out_D, self.graph, self.index.storage_cuda,
+            self.query_cuda, EP_I, EP_D, counters)
+        return out_I, out_D
+
+    def step(self, ef):
+        EP_I, EP_D = self.entries()
+        return self.traverse(ef, EP_I, EP_D)
+
+
+def end_to_end_recall(index, stage, ef, target, k):
+    """Recall of the whole three-stage search at this ef: device candidates,
+    then the host refine on the full-dimension vectors."""
+    from pilotann_amd import kernels, utils
+    out_I, out_D = stage.step(ef)
+    torch.cuda.synchronize()
+    buf_I = out_I.flatten(1).cpu()
+    buf_D = out_D.flatten(1).cpu()
+    top_I = torch.empty(stage.B, k, dtype=torch.long)
+    top_D = torch.empty(stage.B, k, dtype=torch.float)
+    t0 = time.perf_counter()
+    kernels.traverse_refine(
+        top_I, top_D, buf_I, buf_D, buf_I, buf_D,
+        [index.subgraph.indptr, index.subgraph.indices],
+        [index.fullgraph.indptr, index.fullgraph.indices],
+        index.storage, stage.query_rot, ef, index.d_principle)
+    refine_s = time.perf_counter() - t0
+    return utils.recall(top_I, target), refine_s
+
+
+def algorithmic_bytes(counters, B, dp, n_init):
+    """Bytes a search must move, per launch: 4-byte ids, 4-byte floats.
+    query + entries + per expansion (pop id, row pointer) + adjacency entries
+    + per evaluated neighbour (id + dp floats) + results written."""
+    E, A, C, _, R = [int(c) for c in counters]
+    w = 4
+    return (B * (4 * dp + n_init * (w + 4)) + E * 2 * w + A * w
+            + C * (w + 4 * dp) + R * (w + 4))
+
+
+def cpu_baseline(index, stage, ef, EP_I, EP_D, budget_s=15.0):
+    """The host search of the reference (restated in oracle/) on the same
+    subgraph, reduced rows and entries, timed on this box's cores on a sample
+    of the batch sized for about `budget_s` seconds."""
+    import oracle
+    dp = index.d_principle
+    reduced = np.ascontiguousarray(index.storage[:, :dp].numpy())
+    q = np.ascontiguousarray(stage.query_rot[:, :dp].numpy())
+    indptr = index.subgraph.indptr.numpy()
+    indices = index.subgraph.indices.numpy()
+    kk = 4 * ef
+    I = EP_I.cpu().numpy()
+    D = EP_D.cpu().numpy()
+
+    def run(n):
+        out_I = np.empty((n, kk), np.int64)
+        out_D = np.empty((n, kk), np.float32)
+        t0 = time.perf_counter()
+        oracle.traverse_cpu(out_I, out_D, I[:n].copy(), D[:n].copy(), indptr,
+                            indices, reduced, q[:n].copy(), kk)
+        return time.perf_counter() - t0, out_I, out_D
+
+    probe = min(stage.B, 512)
+    run(probe)  # warm-up: thread pool, page faults
+    t_probe, _, _ = run(probe)
+    n = int(min(stage.B, max(probe, probe * budget_s / max(t_probe, 1e-6))))
+    t, out_I, out_D = run(n)
+    return dict(value=n / t, unit='queries/s', cores=oracle.num_threads(),
+                kind='port',
+                sample=f'{n} of {stage.B} queries of the same batch, same '
+                       f'subgraph / reduced rows / entries, ef_search={kk}, '
+                       f'{t:.2f}s'), (out_I, out_D, n)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=20)
+    ap.add_argument('--warmup', type=int, default=3)
+    ap.add_argument('--config', default='c3', choices=sorted(CONFIGS))
+    ap.add_argument('--n-base', type=int, default=None)
+    ap.add_argument('--queries', type=int, default=None)
+    ap.add_argument('--ef', type=int, default=None)
+    ap.add_argument('--no-cpu-baseline', action='store_true')
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
+        print('bench.py: this build measures one GPU; the search shards by '
+              'query batch with no exchange, run it with --gpus 1',
+              file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print('bench.py: no GPU', file=sys.stderr)
+        sys.exit(1)
+
+    cfg = dict(CONFIGS[args.config])
+    if args.n_base:
+        cfg['n'] = args.n_base
+    if args.queries:
+        cfg['queries'] = args.queries
+    device = 'cuda:0'
+    torch.cuda.set_device(0)
+    index, query, target = build_index(cfg, device)
+    stage = Stage(index, query, device)
+    B, k, dp = stage.B, cfg['k'], cfg['dp']
+
+    # pick ef: smallest of the sweep with end-to-end recall@k >= 0.90
+    sweep = []
+    chosen = None
+    for ef in ([args.ef] if args.ef else cfg['ef_sweep']):
+        rec, refine_s = end_to_end_recall(index, stage, ef, target, k)
+        sweep.append(dict(ef=ef, recall=round(rec, 4),
+                          refine_qps=round(B / refine_s, 1)))
+        log(f'[bench] ef={ef} recall@{k}={rec:.4f} host refine {refine_s:.2f}s')
+        if rec >= 0.90:
+            chosen = ef
+            break
+    if chosen is None:
+        chosen = sweep[-1]['ef']
+    ef = chosen
+    recall_at = [s for s in sweep if s['ef'] == ef][0]['recall']
+
+    # work counters of one launch (untimed), then the timed steps
+    EP_I, EP_D = stage.entries()
+    counters = torch.zeros(5, dtype=torch.long, device=device)
+    out_I, out_D = stage.traverse(ef, EP_I, EP_D, counters)
+    torch.cuda.synchronize()
+    counts = counters.cpu().tolist()
+    launch_bytes = algorithmic_bytes(counts, B, dp, EP_I.size(1))
+
+    for _ in range(args.warmup):
+        stage.step(ef)
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True),
+           torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for a, b in ev:
+        EP_I, EP_D = stage.entries()
+        a.record()
+        stage.traverse(ef, EP_I, EP_D)
+        b.record()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = 1e3 * elapsed / args.steps
+    kernel_ms = float(np.mean([a.elapsed_time(b) for a, b in ev]))
+    achieved = launch_bytes / (kernel_ms * 1e-3) / 1e9
+
+    line = {
+        'metric': METRIC,
+        'value': round(B / (ms_per_step * 1e-3), 1),
+        'unit': 'queries/s',
+        'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
+        'ms_per_step': round(ms_per_step, 4),
+        'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
+        'dtype': 'f32', 'data': 'synthetic',
+        'config': {
+            'workload': f'{args.config}: {cfg["n"]} x {cfg["d"]} unit-norm '
+                        f'{cfg["n_centers"]}-component mixture, dp={dp}, '
+                        f'sample_ratio={cfg["ratio"]}, {cfg["graph"]}, '
+                        f'{cfg["entry"]}, {B} queries, top-{k}',
+            'ef': ef, 'recall_at_10': recall_at, 'sweep': sweep,
+            'stage': 'routing_cuda + traverse_cuda (GPU search stage)',
+        },
+        'roofline': {
+            'bound': 'hbm', 'achieved': round(achieved, 1),
+            'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
+            'frac': round(achieved / HBM_PEAK_GBS, 4), 'traffic': None,
+            'kernel': 'traverse_kernel',
+            'kernel_ms': round(kernel_ms, 4),
+            'algorithmic_bytes_per_launch': launch_bytes,
+            'counters': dict(zip(['expanded', 'adjacency_entries',
+                                  'distances', 'admitted', 'result_slots'],
+                                 counts)),
+        },
+    }
+    if not args.no_cpu_baseline:
+        EP_I, EP_D = stage.entries()
+        torch.cuda.synchronize()
+        base, (ref_I, ref_D, n) = cpu_baseline(index, stage, ef, EP_I, EP_D)
+        line['cpu_baseline'] = base
+        same = (np.array_equal(out_D.flatten(1)[:n].cpu().numpy(), ref_D))
+        line['config']['matches_cpu_baseline'] = bool(same)
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == '__main__':
+    main()

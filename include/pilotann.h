@@ -137,6 +137,67 @@ int pa_route(int64_t *router, float *dist, const float *query,
              const float *route_vectors, const float *entry_vectors,
              int64_t batch, int n_routers, int n_leaves, int dp, void *stream);
 
+/* ---- host stages and the chunk pipeline ------------------------------------- */
+
+/*
+ * Replaces `traverse_cpu` (extension/traverse_cpu.cpp:167-257,
+ * pilot_ann/kernels/__init__.py:47-59): one best-first search per query on the
+ * CPU (OpenMP over queries).  Host pointers.  out_* are [batch * k], init_*
+ * [batch * n_init], rows of storage [n_storage * d_model] are addressed by
+ * node id.  Heap size = pa_heap_size(ef_search); at most min(1024,
+ * 2 * ef_search) expansions.
+ */
+int pa_traverse_cpu(int64_t *out_I, float *out_D, int64_t *init_I,
+                    float *init_D, const int64_t *indptr,
+                    const int64_t *indices, const float *storage,
+                    const float *query, int64_t batch, int64_t n_storage,
+                    int d_model, int n_init, int k, int ef_search);
+
+/*
+ * Replaces `traverse_refine` (extension/traverse_cpu.cpp:261-369,
+ * pilot_ann/kernels/__init__.py:78-94).  Host pointers.  init_* [batch *
+ * n_init] hold the device stage's candidates with distances over the first
+ * d_principle coordinates; the remaining coordinates are added to init_D in
+ * place.  Stage 2 (at most two expansions on the subgraph) writes buf_*
+ * [batch * n_buffers], stage 3 (full graph) writes out_* [batch * k].  buf_*
+ * may be the same memory as init_*.
+ */
+int pa_traverse_refine(int64_t *out_I, float *out_D, int64_t *buf_I,
+                       float *buf_D, int64_t *init_I, float *init_D,
+                       const int64_t *sub_indptr, const int64_t *sub_indices,
+                       const int64_t *full_indptr, const int64_t *full_indices,
+                       const float *storage, const float *query, int64_t batch,
+                       int64_t n_storage, int d_model, int d_principle,
+                       int n_init, int n_buffers, int k, int ef_search);
+
+/*
+ * Replaces `pipeline` (extension/pipeline_cpu.cpp:32-145,
+ * pilot_ann/kernels/__init__.py:106-124): splits the batch into chunks, runs
+ * pa_traverse for chunk i+1 and i+2 on two internal streams while
+ * pa_traverse_refine finishes chunk i on the host.
+ *
+ *   topk_I / topk_D [batch * k]: host, out.
+ *   full_* / sub_* : host CSR of the full graph and of the subgraph (global
+ *   ids), storage [n_nodes * d_model] and query [batch * d_model]: host.
+ *   adj, gid, mapping, storage_dev [n_storage * d_principle],
+ *   query_dev [batch * d_principle], init_I / init_D [batch * n_init]: device.
+ *   caller_stream: the stream that produced query_dev / init_*; it is
+ *   synchronised before the first chunk starts (pipeline_cpu.cpp:74-75).
+ *
+ * Blocking.  Device and pinned buffers are kept between calls.  Calls are
+ * serialised by a lock.
+ */
+int pa_pipeline(int64_t *topk_I, float *topk_D, const int64_t *full_indptr,
+                const int64_t *full_indices, const int64_t *sub_indptr,
+                const int64_t *sub_indices, const float *storage,
+                const float *query, const int32_t *adj, const int32_t *gid,
+                const int64_t *mapping, const float *storage_dev,
+                const float *query_dev, const int64_t *init_I,
+                const float *init_D, int64_t batch, int64_t n_nodes,
+                int64_t n_storage, int d_model, int d_principle, int n_init,
+                int n_neighbors, int ef_search, int k, int chunk_size,
+                void *caller_stream);
+
 #ifdef __cplusplus
 }
 #endif

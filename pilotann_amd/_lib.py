@@ -31,10 +31,7 @@ _SIGNATURES = {
     'pa_traverse_refine': (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                                   _vp, _vp, _vp, _vp, _i64, _i64, _int, _int,
                                   _int, _int, _int, _int]),
-    'pa_pipeline': (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
-                           _vp, _vp, _vp, _vp, _vp, _vp,
-                           _i64, _i64, _i64, _int, _int, _int, _int, _int,
-                           _int, _int, _int, _vp]),
+    'pa_pipeline': (_int, [_vp] * 15 + [_i64, _i64, _i64] + [_int] * 7 + [_vp]),
 }
 
 _lib = None

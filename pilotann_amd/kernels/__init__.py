@@ -256,3 +256,155 @@ def entry_distances(query: torch.Tensor, entry_vectors: torch.Tensor):
             query.size(0), 0, entry_vectors.size(0), query.size(-1),
             _stream()), 'pa_route')
     return distances
+
+
+# ---- host stages ------------------------------------------------------------
+
+def traverse_cpu(output_I: torch.Tensor,
+                 output_D: torch.Tensor,
+                 initial_I: torch.Tensor,
+                 initial_D: torch.Tensor,
+                 indptr: torch.Tensor,
+                 indices: torch.Tensor,
+                 storage: torch.Tensor,
+                 query: torch.Tensor,
+                 ef_search: int):
+    """``kernels.traverse_cpu`` (``pilot_ann/kernels/__init__.py:47-59``,
+    checks of ``traverse_cpu.cpp:174-193``)."""
+    _check(query, 'query', 2, torch.float32, False)
+    _check(indptr, 'indptr', 1, torch.int64, False)
+    _check(indices, 'indices', 1, torch.int64, False)
+    _check(storage, 'storage', 2, torch.float32, False)
+    _check(initial_I, 'initial_I', 2, torch.int64, False)
+    _check(initial_D, 'initial_D', 2, torch.float32, False)
+    _check(output_I, 'output_I', 2, torch.int64, False)
+    _check(output_D, 'output_D', 2, torch.float32, False)
+    batch_size, d_model = query.shape
+    _require(storage.size(-1) == d_model, 'storage.size(-1) == d_model')
+    _require(output_I.size(0) == batch_size, 'output_I.size(0) == batch_size')
+    _require(initial_I.size(0) == batch_size,
+             'initial_I.size(0) == batch_size')
+    _require(output_I.size() == output_D.size(),
+             'output_I.sizes() == output_D.sizes()')
+    _require(initial_I.size() == initial_D.size(),
+             'initial_I.sizes() == initial_D.sizes()')
+    _require(ef_search <= 2048, 'ef_search supported')
+    _lib.check(_lib.lib().pa_traverse_cpu(
+        _ptr(output_I), _ptr(output_D), _ptr(initial_I), _ptr(initial_D),
+        _ptr(indptr), _ptr(indices), _ptr(storage), _ptr(query), batch_size,
+        storage.size(0), d_model, initial_I.size(-1), output_I.size(-1),
+        int(ef_search)), 'pa_traverse_cpu')
+
+
+def traverse_refine(output_I: torch.Tensor,
+                    output_D: torch.Tensor,
+                    buffer_I: torch.Tensor,
+                    buffer_D: torch.Tensor,
+                    initial_I: torch.Tensor,
+                    initial_D: torch.Tensor,
+                    subgraph: list,
+                    fullgraph: list,
+                    storage: torch.Tensor,
+                    query: torch.Tensor,
+                    ef_search: int,
+                    d_principle: int):
+    """``kernels.traverse_refine`` (``pilot_ann/kernels/__init__.py:78-94``,
+    checks of ``traverse_cpu.cpp:270-294``).  ``initial_D`` is updated in
+    place with the residual distance."""
+    _require(len(subgraph) == 2, 'subgraph.size() == 2')
+    _require(len(fullgraph) == 2, 'fullgraph.size() == 2')
+    _check(query, 'query', 2, torch.float32, False)
+    _check(storage, 'storage', 2, torch.float32, False)
+    _check(initial_I, 'initial_I', 2, torch.int64, False)
+    _check(initial_D, 'initial_D', 2, torch.float32, False)
+    _check(buffer_I, 'buffer_I', 2, torch.int64, False)
+    _check(buffer_D, 'buffer_D', 2, torch.float32, False)
+    _check(output_I, 'output_I', 2, torch.int64, False)
+    _check(output_D, 'output_D', 2, torch.float32, False)
+    for g in (*subgraph, *fullgraph):
+        _check(g, 'graph', 1, torch.int64, False)
+    batch_size, d_model = query.shape
+    _require(storage.size(-1) == d_model, 'storage.size(-1) == d_model')
+    _require(output_I.size(0) == batch_size, 'output_I.size(0) == batch_size')
+    _require(buffer_I.size(0) == batch_size, 'buffer_I.size(0) == batch_size')
+    _require(initial_I.size(0) == batch_size,
+             'initial_I.size(0) == batch_size')
+    _require(output_I.size() == output_D.size(),
+             'output_I.sizes() == output_D.sizes()')
+    _require(buffer_I.size() == buffer_D.size(),
+             'buffer_I.sizes() == buffer_D.sizes()')
+    _require(initial_I.size() == initial_D.size(),
+             'initial_I.sizes() == initial_D.sizes()')
+    _require(ef_search <= 2048, 'ef_search supported')
+    _lib.check(_lib.lib().pa_traverse_refine(
+        _ptr(output_I), _ptr(output_D), _ptr(buffer_I), _ptr(buffer_D),
+        _ptr(initial_I), _ptr(initial_D), _ptr(subgraph[0]),
+        _ptr(subgraph[1]), _ptr(fullgraph[0]), _ptr(fullgraph[1]),
+        _ptr(storage), _ptr(query), batch_size, storage.size(0), d_model,
+        int(d_principle), initial_I.size(-1), buffer_I.size(-1),
+        output_I.size(-1), int(ef_search)), 'pa_traverse_refine')
+
+
+def pipeline(graph: list,
+             subgraph: list,
+             subgraph_cuda: list,
+             storage: torch.Tensor,
+             storage_cuda: torch.Tensor,
+             query: torch.Tensor,
+             query_cuda: torch.Tensor,
+             initial_I: torch.Tensor,
+             initial_D: torch.Tensor,
+             n_neighbors: int,
+             k: int,
+             ef_search: int,
+             d_principle: int,
+             chunk_size: int):
+    """``kernels.pipeline`` (``pilot_ann/kernels/__init__.py:106-124``, checks
+    of ``pipeline_cpu.cpp:41-58``): device traversal in chunks overlapped
+    with the host refine; returns ``(topk_I[B, k] int64, topk_D[B, k]
+    float32)`` on the CPU."""
+    _require(len(graph) == 2, 'graph.size() == 2')
+    _require(len(subgraph) == 2, 'subgraph.size() == 2')
+    _require(len(subgraph_cuda) == 3, 'subgraph_cuda.size() == 3')
+    _check(query, 'query', 2, torch.float32, False)
+    _check(storage, 'storage', 2, torch.float32, False)
+    _check(graph[0], 'graph[0]', 1, torch.int64, False)
+    _check(graph[1], 'graph[1]', 1, torch.int64, False)
+    _check(subgraph[0], 'subgraph[0]', 1, torch.int64, False)
+    _check(subgraph[1], 'subgraph[1]', 1, torch.int64, False)
+    _check(query_cuda, 'query_cuda', 2, torch.float32, True)
+    _check(storage_cuda, 'storage_cuda', 2, torch.float32, True)
+    _check(subgraph_cuda[0], 'subgraph_cuda[0]', 1, torch.int64, True)
+    _check(subgraph_cuda[1], 'subgraph_cuda[1]', 1, torch.int64, True)
+    _check(subgraph_cuda[2], 'subgraph_cuda[2]', 1, torch.int64, True)
+    _check(initial_I, 'initial_I', 2, torch.int64, True)
+    _check(initial_D, 'initial_D', 2, torch.float32, True)
+    batch_size, d_model = query.shape
+    _require(batch_size % chunk_size == 0, 'batch_size % chunk_size == 0')
+    _require(storage.size(-1) == d_model, 'storage.size(-1) == d_model')
+    _require(query_cuda.size(0) == batch_size,
+             'query_cuda.size(0) == batch_size')
+    _require(query_cuda.size(-1) == d_principle == storage_cuda.size(-1),
+             'query_cuda.size(-1) == d_principle')
+    _require(initial_I.size(0) == batch_size,
+             'initial_I.size(0) == batch_size')
+    _require(initial_I.size() == initial_D.size(),
+             'initial_I.sizes() == initial_D.sizes()')
+    _require(1 <= n_neighbors <= 64, '1 <= n_neighbors <= 64')
+    _require(BEAM_WIDTH * ef_search <= 2048, 'heapq_size supported')
+    prepared = prepare_graph(subgraph_cuda[0], subgraph_cuda[1],
+                             subgraph_cuda[2], storage_cuda.size(0),
+                             n_neighbors)
+    topk_I = torch.empty(batch_size, k, dtype=torch.int64)
+    topk_D = torch.empty(batch_size, k, dtype=torch.float32)
+    with torch.cuda.device(query_cuda.device):
+        _lib.check(_lib.lib().pa_pipeline(
+            _ptr(topk_I), _ptr(topk_D), _ptr(graph[0]), _ptr(graph[1]),
+            _ptr(subgraph[0]), _ptr(subgraph[1]), _ptr(storage), _ptr(query),
+            _ptr(prepared.adj), _ptr(prepared.gid), _ptr(prepared.mapping),
+            _ptr(storage_cuda), _ptr(query_cuda), _ptr(initial_I),
+            _ptr(initial_D), batch_size, prepared.n_nodes,
+            prepared.n_storage, d_model, int(d_principle),
+            initial_I.size(-1), int(n_neighbors), int(ef_search), int(k),
+            int(chunk_size), _stream()), 'pa_pipeline')
+    return topk_I, topk_D

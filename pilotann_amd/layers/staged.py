@@ -1,0 +1,161 @@
+import torch
+from torch import nn
+
+from .. import kernels, utils
+from .entry import IndexEntry
+
+
+class GraphModule(nn.Module):
+    """CSR graph as two int64 buffers (``layers/staged.py:6-17``)."""
+
+    def __init__(self, indptr, indices):
+        super().__init__()
+        self.register_buffer(
+            'indptr', torch.as_tensor(indptr, dtype=torch.long).contiguous())
+        self.register_buffer(
+            'indices', torch.as_tensor(indices, dtype=torch.long).contiguous())
+
+
+class IndexStaged(nn.Module):
+    """Three-stage index, interface of ``pilot_ann/layers/staged.py:20-228``:
+    device traversal of the sampled subgraph on the first ``d_principle``
+    rotated coordinates, then the host refine on the subgraph and on the full
+    graph in full dimension.
+
+    ``seed`` and ``build_device`` are additions: every random choice of the
+    build is seeded, and the build-time matrix products run where
+    ``build_device`` says (the search-time split is the reference's).
+    """
+
+    def __init__(self, d_model: int, d_principle: int, sample_ratio: float,
+                 graph_method: str = 'nsw32', entry_method: str = 'random32',
+                 seed: int = 0, build_device: str = 'cpu'):
+        super().__init__()
+        assert d_principle <= d_model
+        self.d_model = d_model
+        self.d_principle = d_principle
+        self.sample_ratio = sample_ratio
+        self.graph_method = graph_method
+        self.entry_method = entry_method
+        self.seed = seed
+        self.build_device = build_device
+        self.cuda_device = None
+        for graph_type in ['nsw', 'nsg']:
+            if graph_method.startswith(graph_type):
+                self.graph_type = graph_type
+                self.n_neighbors = int(graph_method.removeprefix(graph_type))
+                break
+        else:
+            raise NotImplementedError
+        self.entry = IndexEntry(d_model=d_principle, method=entry_method,
+                                seed=seed + 3)
+        self.storage_cuda = None
+        self.subgraph_cuda = None
+        self.mapping_cuda = None
+
+    # -- checkpoint: layers/staged.py:59-122 ---------------------------------
+    @classmethod
+    def load(cls, ckpt_file):
+        checkpoint = torch.load(ckpt_file, weights_only=True)
+        state = checkpoint['state_dict']
+        config = checkpoint['config']
+        index = cls(d_model=config['d_model'],
+                    d_principle=config['d_principle'],
+                    graph_method=config['graph_method'],
+                    entry_method=config['entry_method'], sample_ratio=-1.0)
+        for name in ['VT', 'storage', 'mapping', 'nodelist']:
+            index.register_buffer(name, state[name])
+        index.register_module('subgraph', GraphModule(
+            state['subgraph.indptr'], state['subgraph.indices']))
+        index.register_module('fullgraph', GraphModule(
+            state['fullgraph.indptr'], state['fullgraph.indices']))
+        for name in ['entry_nodes', 'entry_vectors', 'route_vectors']:
+            if 'entry.' + name in state:
+                index.entry.register_buffer(name, state['entry.' + name])
+        return index
+
+    def dump(self):
+        keep = ('VT', 'storage', 'mapping', 'nodelist', 'subgraph.',
+                'fullgraph.', 'entry.')
+        return {
+            'config': {
+                'd_model': self.d_model,
+                'd_principle': self.d_principle,
+                'graph_method': self.graph_method,
+                'entry_method': self.entry_method,
+            },
+            'state_dict': {k: v for k, v in self.state_dict().items()
+                           if k.startswith(keep)},
+        }
+
+    # -- device residency: layers/staged.py:124-139 ---------------------------
+    def to(self, device):
+        """Copies what the device stage needs: entries, mapping, the subgraph
+        and the first ``d_principle`` coordinates of the sampled rows; the
+        search form of the subgraph is prepared here, once."""
+        self.cuda_device = device
+        self.entry.to(device=device)
+        self.mapping_cuda = self.mapping.to(device=device)
+        self.subgraph_cuda = GraphModule(self.subgraph.indptr,
+                                         self.subgraph.indices).to(device)
+        rows = torch.index_select(self.storage, 0, self.nodelist)
+        self.storage_cuda = rows[:, :self.d_principle].contiguous().to(device)
+        if torch.device(device).type == 'cuda':
+            kernels.prepare_graph(
+                self.subgraph_cuda.indptr, self.subgraph_cuda.indices,
+                self.mapping_cuda, self.storage_cuda.size(0), self.n_neighbors)
+        return self
+
+    # -- build: layers/staged.py:141-189 --------------------------------------
+    def train(self, x: torch.Tensor):
+        assert x.dim() == 2
+        assert x.size(-1) == self.d_model
+        assert 0.0 < self.sample_ratio <= 1.0
+        dev = self.build_device
+        half = torch.float16 if torch.device(dev).type == 'cuda' else None
+
+        print('svd', self.d_principle)
+        xr, V = utils.svd(x.to(dev), max_size=10_000_000, seed=self.seed)
+        self.register_buffer('storage', xr.cpu().contiguous())
+        self.register_buffer('VT', V.T.contiguous().cpu())
+
+        print('build', self.graph_type)
+        graph = utils.graph_init(xr, graph_type=self.graph_type,
+                                 n_neighbors=self.n_neighbors,
+                                 compute_dtype=half)
+        self.register_module('fullgraph', GraphModule(graph[0], graph[1]))
+
+        print('sampling', self.sample_ratio)
+        sub = utils.subgraph_init(
+            indptr=graph[0], indices=graph[1], storage=xr,
+            graph_type=self.graph_type,
+            n_samples=round(self.sample_ratio * x.size(0)),
+            n_neighbors=self.n_neighbors, seed=self.seed + 1,
+            compute_dtype=half)
+        self.register_module('subgraph', GraphModule(sub[0], sub[1]))
+        self.register_buffer('nodelist', sub[2].contiguous())
+        self.register_buffer('mapping', sub[3].contiguous())
+
+        self.entry.train(self.storage[:, :self.d_principle])
+        return self
+
+    # -- search: layers/staged.py:191-228 -------------------------------------
+    @torch.no_grad()
+    def search(self, query: torch.Tensor, k: int, ef_search: int,
+               chunk_size: int = 128):
+        assert query.dim() == 2
+        query = torch.matmul(query, self.VT.T).contiguous()
+        query_cuda = query[:, :self.d_principle].contiguous().to(
+            device=self.cuda_device)
+        EP_I, EP_D = self.entry.search(query_cuda)
+        return kernels.pipeline(
+            graph=[self.fullgraph.indptr, self.fullgraph.indices],
+            storage=self.storage,
+            subgraph=[self.subgraph.indptr, self.subgraph.indices],
+            subgraph_cuda=[self.subgraph_cuda.indptr,
+                           self.subgraph_cuda.indices, self.mapping_cuda],
+            storage_cuda=self.storage_cuda, query=query,
+            query_cuda=query_cuda, initial_I=EP_I.contiguous(),
+            initial_D=EP_D.contiguous(), k=k, n_neighbors=self.n_neighbors,
+            ef_search=ef_search, d_principle=self.d_principle,
+            chunk_size=chunk_size)

@@ -137,22 +137,23 @@ def graph_init(x: torch.Tensor, graph_type: str, n_neighbors: int,
 
 
 def graph_sampling(indptr: torch.Tensor, indices: torch.Tensor,
-                   n_samples: int, n_hops: int, seed: int = 0):
+                   n_samples: int, n_hops: int, seed: int = 0,
+                   device: str = 'cpu'):
     """Seeded version of ``extension/sampling_cpu.cpp:5-65``: random seed
     nodes, each with its ``n_hops`` neighbourhood, are added in a fixed random
     order until at least ``n_samples`` nodes are in.  Returns the sorted
     ``nodelist`` and ``mapping`` (global id → position in nodelist, else -1).
     """
-    indptr = torch.as_tensor(indptr, dtype=torch.long)
-    indices = torch.as_tensor(indices, dtype=torch.long)
+    indptr = torch.as_tensor(indptr, dtype=torch.long).to(device)
+    indices = torch.as_tensor(indices, dtype=torch.long).to(device)
     n = indptr.numel() - 1
     g = torch.Generator().manual_seed(seed)
-    order = torch.randperm(n, generator=g)
+    order = torch.randperm(n, generator=g).to(device)
     row_of_edge = torch.repeat_interleave(
-        torch.arange(n), indptr[1:] - indptr[:-1])
+        torch.arange(n, device=device), indptr[1:] - indptr[:-1])
 
     def closure(m: int):
-        mark = torch.zeros(n, dtype=torch.bool)
+        mark = torch.zeros(n, dtype=torch.bool, device=device)
         mark[order[:m]] = True
         for _ in range(n_hops):
             hit = indices[mark[row_of_edge]]
@@ -166,7 +167,7 @@ def graph_sampling(indptr: torch.Tensor, indices: torch.Tensor,
             hi = mid
         else:
             lo = mid + 1
-    nodelist = torch.nonzero(closure(lo)).flatten()
+    nodelist = torch.nonzero(closure(lo)).flatten().cpu()
     mapping = torch.full((n,), -1, dtype=torch.long)
     mapping[nodelist] = torch.arange(nodelist.numel())
     return nodelist, mapping
@@ -182,7 +183,7 @@ def subgraph_init(indptr: torch.Tensor, indices: torch.Tensor,
     (the reference turns it into the last sampled node, ``graphs.py:123-126``;
     both end a row's useful part the same way for the search)."""
     nodelist, mapping = graph_sampling(indptr, indices, n_samples, n_hops,
-                                       seed=seed)
+                                       seed=seed, device=storage.device)
     sub = storage[nodelist.to(storage.device)]
     sg_indptr, sg_indices = graph_init(sub, graph_type, n_neighbors,
                                        compute_dtype=compute_dtype)

@@ -4,23 +4,27 @@ import torch
 
 def gaussian_mixture(n: int, d: int, n_centers: int, sigma: float, seed: int,
                      normalize: bool = False, device: str = 'cpu',
-                     center_seed: int = None):
+                     center_seed: int = None, decay: float = 0.0):
     """``n`` points of an isotropic Gaussian mixture: centres ~ N(0, I_d),
     a uniformly drawn centre plus ``sigma``·N(0, I_d) per point; optionally
     projected onto the unit sphere.  ``center_seed`` fixes the centres apart
     from the points, so that queries (another ``seed``) share the base set's
-    mixture."""
+    mixture.  With ``decay`` > 0 coordinate j (of centres and noise alike)
+    is scaled by (1 + j)^(-decay): a power-law spectrum like that of learned
+    embeddings, where the leading SVD coordinates carry most of a distance;
+    ``decay`` = 0 is the isotropic mixture."""
     gc = torch.Generator(device='cpu').manual_seed(
         seed if center_seed is None else center_seed)
     centers = torch.randn(n_centers, d, generator=gc)
     g = torch.Generator(device='cpu').manual_seed(seed + 7919)
     which = torch.randint(high=n_centers, size=[n], generator=g)
     out = torch.empty(n, d, device=device)
+    scale = torch.arange(1, d + 1, dtype=torch.float32).pow(-decay).to(device)
     centers = centers.to(device)
     for lo in range(0, n, 131072):
         hi = min(n, lo + 131072)
         noise = torch.randn(hi - lo, d, generator=g).to(device)
-        out[lo:hi] = centers[which[lo:hi].to(device)] + sigma * noise
+        out[lo:hi] = (centers[which[lo:hi].to(device)] + sigma * noise) * scale
     if normalize:
         out = torch.nn.functional.normalize(out, dim=-1)
     return out

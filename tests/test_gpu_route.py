@@ -14,7 +14,8 @@ pytestmark = pytest.mark.gpu
                                      (32, 32, 64, 1023), (64, 64, 128, 2500),
                                      (40, 96, 32, 333)])
 def test_routing_matches_oracle(R, L, d, B, device):
-    x = utils.gaussian_mixture(20000, d, 32, 0.5, seed=R + L)
+    n = max(20000, 2 * min(1024, R * R) * L)
+    x = utils.gaussian_mixture(n, d, 32, 0.5, seed=R + L)
     q = utils.gaussian_mixture(B, d, 32, 0.5, seed=99, center_seed=R + L)
     route_vectors, entry_nodes = utils.router_init(x, None, R, L, seed=1)
     entry_vectors = x[entry_nodes].contiguous()
