@@ -13,6 +13,7 @@ line is printed; `value` is queries per second of that step.
                     [--n-base N] [--queries B] [--ef EF] [--no-cpu-baseline]
 """
 import argparse
+import contextlib
 import json
 import os
 import sys
@@ -61,7 +62,8 @@ def build_index(cfg, device):
                         sample_ratio=cfg['ratio'], graph_method=cfg['graph'],
                         entry_method=cfg['entry'], seed=cfg['seed'],
                         build_device=device)
-    index.train(x)
+    with contextlib.redirect_stdout(sys.stderr):  # keep stdout to the JSON line
+        index.train(x)
     del x
     torch.cuda.empty_cache()
     index.to(device)

@@ -35,7 +35,11 @@ def _run(cmd, verbose):
     subprocess.run(cmd, check=True)
 
 
-def build(verbose: bool = False) -> str:
+def build(verbose: bool = False, output: str = LIB,
+          extra_hip_flags=()) -> str:
+    """Compile everything and link ``output`` (default: the library the
+    loader uses).  ``extra_hip_flags`` are added to the device compiles, e.g.
+    ``-DPA_PHASE_TIMERS`` for a tuning build written elsewhere."""
     include = os.path.join(ROOT, 'include')
     objects = []
     for name in HIP_SOURCES:
@@ -43,8 +47,8 @@ def build(verbose: bool = False) -> str:
         if not os.path.exists(src):
             continue
         obj = os.path.join(CSRC, name + '.o')
-        _run(['hipcc', *HIP_FLAGS, '-I', include, '-c', src, '-o', obj],
-             verbose)
+        _run(['hipcc', *HIP_FLAGS, *extra_hip_flags, '-I', include, '-c', src,
+              '-o', obj], verbose)
         objects.append(obj)
     for name in CXX_SOURCES:
         src = os.path.join(CSRC, name)
@@ -53,11 +57,11 @@ def build(verbose: bool = False) -> str:
         obj = os.path.join(CSRC, name + '.o')
         _run(['g++', *CXX_FLAGS, '-I', include, '-c', src, '-o', obj], verbose)
         objects.append(obj)
-    _run(['hipcc', '--offload-arch=gfx950', '-shared', '-fPIC', '-o', LIB,
+    _run(['hipcc', '--offload-arch=gfx950', '-shared', '-fPIC', '-o', output,
           *objects, '-lgomp', '-lpthread'], verbose)
     for obj in objects:
         os.remove(obj)
-    return LIB
+    return output
 
 
 if __name__ == '__main__':

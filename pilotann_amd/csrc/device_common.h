@@ -52,37 +52,58 @@ __device__ __forceinline__ float wave_max(float x) {
 // Squared L2 between a query held in LDS and one storage row, in the order of
 // the reference's host code (extension/inc/distance.h:31-55): element j of
 // every group of eight goes to accumulator j with one FMA, the eight
-// accumulators are then added left to right.  Two adjacent lanes share a row:
-// the even lane (half 0) owns accumulators 0..3, the odd lane (half 1) 4..7;
-// `row` and `qv` already point at the lane's half of the first group.  The
-// even lane returns the distance; every lane of the wavefront must call this
-// (the exchange between the two lanes is a DPP move), lanes without a row
-// pass active = false.
+// accumulators are then added left to right.  Four adjacent lanes (a quad)
+// share a row: lane a of the quad owns accumulators 2a and 2a + 1 and streams
+// its 8 bytes of every 32-byte group, so all loads of a row are in flight at
+// once in 2 * dp / 8 registers.  `row` and `qv` already point at the lane's
+// pair of the first group.  Lane 0 of the quad returns the distance; every
+// lane of the wavefront must call this (the exchange inside the quad is a DPP
+// move), lanes without a row pass active = false.
+constexpr int kLanesPerRow = 4;
+constexpr int kRowsPerPass = kWave / kLanesPerRow;
+
 template <int DP8>
-__device__ __forceinline__ float pair_square_dist(const float4 *row,
-                                                  const float4 *qv, int groups,
+__device__ __forceinline__ float quad_square_dist(const float2 *row,
+                                                  const float2 *qv, int groups,
                                                   bool active) {
-    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    float a0 = 0.f, a1 = 0.f;
     if (active) {
-        const int n = DP8 ? DP8 : groups;
-#pragma unroll 8
-        for (int t = 0; t < n; ++t) {
-            const float4 x = row[2 * t];
-            const float4 y = qv[2 * t];
-            const float d0 = y.x - x.x, d1 = y.y - x.y;
-            const float d2 = y.z - x.z, d3 = y.w - x.w;
-            acc.x = fmaf(d0, d0, acc.x);
-            acc.y = fmaf(d1, d1, acc.y);
-            acc.z = fmaf(d2, d2, acc.z);
-            acc.w = fmaf(d3, d3, acc.w);
+        if (DP8) {
+            // all loads of the row first; the query is then read from LDS
+            // four groups at a time (the fences keep the compiler from
+            // hoisting those reads, which would double the live registers)
+            float2 x[DP8 ? DP8 : 1];
+#pragma unroll
+            for (int t = 0; t < DP8; ++t) x[t] = row[4 * t];
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int t = 0; t < DP8; ++t) {
+                const float2 y = qv[4 * t];
+                const float d0 = y.x - x[t].x, d1 = y.y - x[t].y;
+                a0 = fmaf(d0, d0, a0);
+                a1 = fmaf(d1, d1, a1);
+                if ((t & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+            }
+        } else {
+#pragma unroll 4
+            for (int t = 0; t < groups; ++t) {
+                const float2 x = row[4 * t];
+                const float2 y = qv[4 * t];
+                const float d0 = y.x - x.x, d1 = y.y - x.y;
+                a0 = fmaf(d0, d0, a0);
+                a1 = fmaf(d1, d1, a1);
+            }
         }
     }
-    float s = ((acc.x + acc.y) + acc.z) + acc.w;
-    const float o0 = dpp_f<0xF5, 0xF>(acc.x);  // quad_perm [1,1,3,3]
-    const float o1 = dpp_f<0xF5, 0xF>(acc.y);
-    const float o2 = dpp_f<0xF5, 0xF>(acc.z);
-    const float o3 = dpp_f<0xF5, 0xF>(acc.w);
-    return (((s + o0) + o1) + o2) + o3;
+    // accumulators 0..7 left to right: lane 0 has (0, 1), lane 1 (2, 3), ...
+    float s = a0 + a1;
+    s += dpp_f<0x55, 0xF>(a0);  // quad_perm [1,1,1,1]
+    s += dpp_f<0x55, 0xF>(a1);
+    s += dpp_f<0xAA, 0xF>(a0);  // quad_perm [2,2,2,2]
+    s += dpp_f<0xAA, 0xF>(a1);
+    s += dpp_f<0xFF, 0xF>(a0);  // quad_perm [3,3,3,3]
+    s += dpp_f<0xFF, 0xF>(a1);
+    return s;
 }
 
 }  // namespace pa

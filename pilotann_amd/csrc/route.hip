@@ -96,7 +96,7 @@ __global__ __launch_bounds__(kWave) void route_score_kernel(
 }
 
 // One wavefront per query: squared distances to the n_leaves vectors of the
-// query's group, 32 leaves per pass, two lanes per leaf.
+// query's group, 16 leaves per pass, four lanes per leaf.
 template <int DP8>
 __global__ __launch_bounds__(256) void leaf_dist_kernel(
     const float *__restrict__ query, const float *__restrict__ entry_vectors,
@@ -113,15 +113,15 @@ __global__ __launch_bounds__(256) void leaf_dist_kernel(
     if (q >= batch) return;
     const int64_t group = router ? router[q] : 0;
     const float *leaves = entry_vectors + (size_t)group * n_leaves * dp;
-    const int pair = lane >> 1, half = lane & 1;
-    const float4 *qq = reinterpret_cast<const float4 *>(qv) + half;
-    for (int base = 0; base < n_leaves; base += 32) {
-        const int l = base + pair;
+    const int quad = lane >> 2, part = lane & 3;
+    const float2 *qq = reinterpret_cast<const float2 *>(qv) + part;
+    for (int base = 0; base < n_leaves; base += kRowsPerPass) {
+        const int l = base + quad;
         const bool active = l < n_leaves;
-        const float4 *row =
-            reinterpret_cast<const float4 *>(leaves + (size_t)(active ? l : 0) * dp) + half;
-        const float s = pair_square_dist<DP8>(row, qq, dp >> 3, active);
-        if (active && half == 0) dist[(size_t)q * n_leaves + l] = s;
+        const float2 *row =
+            reinterpret_cast<const float2 *>(leaves + (size_t)(active ? l : 0) * dp) + part;
+        const float s = quad_square_dist<DP8>(row, qq, dp >> 3, active);
+        if (active && part == 0) dist[(size_t)q * n_leaves + l] = s;
     }
 }
 

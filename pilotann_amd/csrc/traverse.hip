@@ -4,8 +4,10 @@
 // for step, what the reference's host search does for that query
 // (extension/traverse_cpu.cpp:12-163):
 //   * the open list is the same array heap, with the same sift rules
-//     (extension/inc/heapq.cuh:13-88), kept in LDS and advanced by the whole
-//     wavefront in lock step (uniform control flow, lane 0 stores);
+//     (extension/inc/heapq.cuh:13-88): its top eight levels sit in registers
+//     (one node per lane, read with v_readlane), the rest in LDS, and the
+//     whole wavefront advances it in lock step (uniform control flow, walks
+//     unrolled by level, scalar integer compares);
 //   * the result list is the exact set of the H best distances seen so far —
 //     what the reference's result heap holds — spread over registers,
 //     ceil(H/64) entries per lane;
@@ -13,12 +15,12 @@
 //     slice of a pooled HBM bitmask, tested and set with one atomic OR per
 //     neighbour;
 //   * a distance is the reference's eight-accumulator FMA sum
-//     (extension/inc/distance.h:31-55) bit for bit: two lanes share a row,
-//     the even lane owns accumulators 0..3 and the odd lane 4..7, each lane
-//     streams its half of every 8-float group with 16-byte loads.
+//     (extension/inc/distance.h:31-55) bit for bit: four lanes share a row,
+//     lane a of the quad owns accumulators 2a and 2a+1 and streams its 8
+//     bytes of every 32-byte group.
 // Expansion of a node therefore costs one coalesced row of neighbour ids, one
 // atomic per neighbour and one coalesced 4*dp-byte row per unvisited
-// neighbour, 32 rows in flight per pass.
+// neighbour, 16 rows in flight per pass.
 #include <hip/hip_runtime.h>
 #include <math.h>
 #include <stdint.h>
@@ -33,70 +35,200 @@ namespace {
 constexpr int kSlotAlignWords = 256;   // bitmask slice: multiple of 1 KiB
 constexpr int kWorkCounterBytes = 256; // head of the workspace
 
-// ---- open list: heapq.cuh on LDS -------------------------------------------
-
-__device__ __forceinline__ void open_put(float *key, int *val, int at, float k,
-                                         int v, int lane) {
-    if (lane == 0) {
-        key[at] = k;
-        val[at] = v;
-    }
+// ---- open list: heapq.cuh, top of the heap in registers ----------------------
+//
+// The reference's open list is an array heap of 2H cells with the sift rules
+// of extension/inc/heapq.cuh:13-88.  Here node i of that array is node
+// j = i + 1 (children 2j and 2j + 1), level L holds j in [2^L, 2^(L+1)).
+//
+// Levels 0..7 live in registers, one node per lane: bank A levels 0..5 (node j
+// in lane j), bank B level 6 (lane j - 64), banks C and D the left and right
+// children of level 7 (lane (j - 128) / 2), so a sibling pair is always two
+// v_readlane of known registers.  Deeper nodes sit in LDS at [j - 256], a
+// sibling pair per aligned 8 bytes.  Keys are kept as order-preserving
+// integers (float_to_key) so that every comparison of a walk is a scalar
+// integer compare.  All lanes run the same, uniform, control flow; the walks
+// are unrolled by level so that each level is a dozen instructions.  After
+// each operation the heap is, cell for cell, the reference's.
+__device__ __forceinline__ int float_to_key(float x) {
+    const int b = __float_as_int(x);
+    return b ^ ((b >> 31) & 0x7fffffff);
+}
+__device__ __forceinline__ float key_to_float(int k) {
+    return __int_as_float(k ^ ((k >> 31) & 0x7fffffff));
 }
 
-// heapq.cuh:37-45 with the sift of :13-29: the root leaves, (inf, -1) sinks
-// along the smaller child (left on ties) until it is not larger than it.
-__device__ __forceinline__ void open_pop(float *key, int *val, int size,
-                                         int lane, float &out_k, int &out_v) {
-    out_k = uni(key[0]);
-    out_v = uni(val[0]);
-    int at = 0;
-    for (;;) {
-        int c = 2 * at + 1;
-        if (c >= size) break;
-        float ck = uni(key[c]);
-        int cv = uni(val[c]);
-        if (c + 1 < size) {
-            float rk = uni(key[c + 1]);
-            int rv = uni(val[c + 1]);
-            if (rk < ck) ck = rk, cv = rv, c += 1;
+// c + (a != b) on the scalar unit (the compiler routes the boolean of a
+// uniform compare through a vector register otherwise).
+__device__ __forceinline__ int add_if_ne(int c, int a, int b) {
+    int r;
+    asm("s_cmp_lg_u32 %1, %2\n\ts_addc_u32 %0, %3, 0"
+        : "=s"(r)
+        : "s"(a), "s"(b), "s"(c)
+        : "scc");
+    return r;
+}
+
+constexpr int floor_log2(int x) { return x <= 1 ? 0 : 1 + floor_log2(x >> 1); }
+
+template <int H>
+struct OpenList {
+    static constexpr int kSize = 2 * H;           // cells of the reference heap
+    static constexpr int kDepth = floor_log2(kSize);  // deepest level
+    static constexpr int kRegNodes = 256;
+    static constexpr int kLdsCells = kSize + 2 > kRegNodes ? kSize + 2 - kRegNodes : 0;
+    static constexpr int kInf = 0x7f800000;       // float_to_key(+inf)
+    int Ak, Av, Bk, Bv, Ck, Cv, Dk, Dv;
+    int *lk;  // node j >= 256 at [j - 256]
+    int *lv;
+
+    __device__ __forceinline__ static int rl(int x, int l) {
+        return __builtin_amdgcn_readlane(x, l);
+    }
+    // storage class of a level: 0 bank A, 1 bank B, 2 banks C/D, 3 LDS
+    __device__ __forceinline__ static constexpr int kind(int level) {
+        return level <= 5 ? 0 : level == 6 ? 1 : level == 7 ? 2 : 3;
+    }
+
+    __device__ __forceinline__ void reset(int lane) {
+        Ak = Bk = Ck = Dk = kInf;
+        Av = Bv = Cv = Dv = -1;
+        for (int i = lane; i < kLdsCells; i += kWave) lk[i] = kInf, lv[i] = -1;
+    }
+
+    // keys (and values) of the sibling pair (c, c + 1), c even, of a level.
+    // KIND and VALS are constants once the level loops are unrolled.
+    __device__ __forceinline__ void pair(const int KIND, const bool VALS, int c,
+                                         int &ka, int &kb, int &va,
+                                         int &vb) const {
+        if (KIND == 0) {
+            ka = rl(Ak, c), kb = rl(Ak, c + 1);
+            if (VALS) va = rl(Av, c), vb = rl(Av, c + 1);
+        } else if (KIND == 1) {
+            const int l = c - 64;
+            ka = rl(Bk, l), kb = rl(Bk, l + 1);
+            if (VALS) va = rl(Bv, l), vb = rl(Bv, l + 1);
+        } else if (KIND == 2) {
+            const int l = (c - 128) >> 1;
+            ka = rl(Ck, l), kb = rl(Dk, l);
+            if (VALS) va = rl(Cv, l), vb = rl(Dv, l);
+        } else {
+            const int2 k2 = *reinterpret_cast<const int2 *>(lk + (c - kRegNodes));
+            if (VALS) {
+                const int2 v2 = *reinterpret_cast<const int2 *>(lv + (c - kRegNodes));
+                va = uni(v2.x), vb = uni(v2.y);
+            }
+            ka = uni(k2.x), kb = uni(k2.y);
         }
-        if (INFINITY <= ck) break;
-        open_put(key, val, at, ck, cv, lane);
-        at = c;
     }
-    open_put(key, val, at, INFINITY, -1, lane);
-    wave_sync();
-}
-
-// heapq.cuh:47-77: walk to a leaf through the larger child (left on ties),
-// overwrite it when the new key is strictly smaller, let the new entry rise.
-__device__ __forceinline__ void open_replace(float *key, int *val, int size,
-                                             float k, int v, int lane) {
-    int at = 0;
-    float leaf = uni(key[0]);
-    for (;;) {
-        int c = 2 * at + 1;
-        if (c >= size) break;
-        float ck = uni(key[c]);
-        if (c + 1 < size) {
-            float rk = uni(key[c + 1]);
-            if (rk > ck) ck = rk, c += 1;
+    __device__ __forceinline__ int val_of(const int KIND, int j) const {
+        if (KIND == 0) return rl(Av, j);
+        if (KIND == 1) return rl(Bv, j - 64);
+        if (KIND == 2) {
+            const int l = (j - 128) >> 1;
+            return (j & 1) ? rl(Dv, l) : rl(Cv, l);
         }
-        at = c;
-        leaf = ck;
+        return uni(lv[j - kRegNodes]);
     }
-    if (k >= leaf) return;
-    while (at > 0) {
-        int up = (at - 1) >> 1;
-        float pk = uni(key[up]);
-        if (pk <= k) break;
-        int pv = uni(val[up]);
-        open_put(key, val, at, pk, pv, lane);
-        at = up;
+    __device__ __forceinline__ void put(const int KIND, int j, int k, int v,
+                                        int lane) {
+        if (KIND == 0) {
+            const bool mine = lane == j;
+            Ak = mine ? k : Ak, Av = mine ? v : Av;
+        } else if (KIND == 1) {
+            const bool mine = lane == j - 64;
+            Bk = mine ? k : Bk, Bv = mine ? v : Bv;
+        } else if (KIND == 2) {
+            const bool mine = lane == ((j - 128) >> 1);
+            if (j & 1) {
+                Dk = mine ? k : Dk, Dv = mine ? v : Dv;
+            } else {
+                Ck = mine ? k : Ck, Cv = mine ? v : Cv;
+            }
+        } else if (lane == 0) {
+            lk[j - kRegNodes] = k, lv[j - kRegNodes] = v;
+        }
     }
-    open_put(key, val, at, k, v, lane);
-    wave_sync();
-}
+
+    // heapq.cuh:37-45 with the sift of :13-29: the root leaves, (inf, -1)
+    // sinks along the smaller child (left on ties) while that child is finite.
+    // Levels 1..kDepth-1 are complete; on level kDepth only nodes up to kSize
+    // exist, and node kSize has no sibling.
+    __device__ __forceinline__ void pop(int lane, float &out_k, int &out_v) {
+        out_k = key_to_float(rl(Ak, 1));
+        out_v = rl(Av, 1);
+        int j = 1;
+#pragma unroll
+        for (int L = 1; L <= kDepth; ++L) {
+            const int c = 2 * j;
+            int ka, kb, va, vb;
+            if (L == kDepth) {
+                if (c > kSize) break;
+                pair(kind(L), true, c, ka, kb, va, vb);
+                kb = c == kSize ? ka : kb;
+            } else {
+                pair(kind(L), true, c, ka, kb, va, vb);
+            }
+            const int ck = min(ka, kb);
+            if (ck >= kInf) {
+                put(kind(L - 1), j, kInf, -1, lane);
+                wave_sync();
+                return;
+            }
+            put(kind(L - 1), j, ck, ck != ka ? vb : va, lane);
+            j = add_if_ne(c, ck, ka);
+            if (L == kDepth) {
+                put(kind(L), j, kInf, -1, lane);
+                wave_sync();
+                return;
+            }
+        }
+        put(kind(kDepth - 1), j, kInf, -1, lane);
+        wave_sync();
+    }
+
+    // heapq.cuh:47-77: walk to a leaf through the larger child (left on
+    // ties), overwrite it when the new key is strictly smaller, let the new
+    // entry rise.  The walk keeps the keys it passes, so the rise needs no
+    // further key reads.
+    __device__ __forceinline__ void replace(float key, int v, int lane) {
+        const int k = float_to_key(key);
+        int pj[kDepth + 1], pk[kDepth + 1];
+        pj[0] = 1, pk[0] = rl(Ak, 1);
+        int deepest = kDepth;
+#pragma unroll
+        for (int L = 1; L <= kDepth; ++L) {
+            const int c = 2 * pj[L - 1];
+            int ka, kb, va, vb;
+            if (L == kDepth) {
+                if (c > kSize) {
+                    deepest = kDepth - 1;
+                    pj[L] = 0, pk[L] = 0;
+                    break;
+                }
+                pair(kind(L), false, c, ka, kb, va, vb);
+                kb = c == kSize ? ka : kb;
+            } else {
+                pair(kind(L), false, c, ka, kb, va, vb);
+            }
+            pk[L] = max(ka, kb);
+            pj[L] = add_if_ne(c, pk[L], ka);
+        }
+        if (k >= (deepest == kDepth ? pk[kDepth] : pk[kDepth - 1])) return;
+#pragma unroll
+        for (int L = kDepth; L >= 1; --L) {
+            if (L == kDepth && deepest != kDepth) continue;
+            if (pk[L - 1] <= k) {
+                put(kind(L), pj[L], k, v, lane);
+                wave_sync();
+                return;
+            }
+            put(kind(L), pj[L], pk[L - 1], val_of(kind(L - 1), pj[L - 1]), lane);
+        }
+        put(0, 1, k, v, lane);
+        wave_sync();
+    }
+};
 
 // ---- result list: the H smallest distances, S entries per lane --------------
 //
@@ -149,23 +281,23 @@ struct Results {
 // ---- distances ---------------------------------------------------------------
 
 // Squared L2 from the query (LDS) to the storage rows listed in cand_id[0..n),
-// written to cand_key.  Lane 2p and 2p+1 share row p of each group of 32.
+// written to cand_key: 16 rows per pass, four lanes per row.
 template <int DP8>
 __device__ __forceinline__ void eval_rows(const float *__restrict__ storage,
                                           const float *qv, const int *cand_id,
                                           float *cand_key, int n, int dp,
                                           int lane) {
-    const int pair = lane >> 1, half = lane & 1;
-    const float4 *qq = reinterpret_cast<const float4 *>(qv) + half;
-    for (int base = 0; base < n; base += 32) {
-        const int c = base + pair;
+    const int quad = lane >> 2, part = lane & 3;
+    const float2 *qq = reinterpret_cast<const float2 *>(qv) + part;
+    for (int base = 0; base < n; base += kRowsPerPass) {
+        const int c = base + quad;
         const bool active = c < n;
-        const float4 *row = reinterpret_cast<const float4 *>(storage);
+        const float2 *row = reinterpret_cast<const float2 *>(storage);
         if (active)
-            row = reinterpret_cast<const float4 *>(
-                      storage + (size_t)cand_id[c] * (size_t)dp) + half;
-        const float s = pair_square_dist<DP8>(row, qq, dp >> 3, active);
-        if (active && half == 0) cand_key[c] = s;
+            row = reinterpret_cast<const float2 *>(
+                      storage + (size_t)cand_id[c] * (size_t)dp) + part;
+        const float s = quad_square_dist<DP8>(row, qq, dp >> 3, active);
+        if (active && part == 0) cand_key[c] = s;
     }
 }
 
@@ -185,19 +317,37 @@ struct TraverseArgs {
     int *work_counter;
     unsigned long long *counters;
     int batch, n_nodes, n_storage, dp, n_init, k, H, deg, max_iter;
-    int words_per_slot, sort_n;
+    int words_per_slot, sort_n, lds_cells;
 };
 
 __global__ void reset_work_counter(int *counter) { *counter = 0; }
 
-template <int S, int DP8>
+// Optional per-phase cycle tally for tuning builds (-DPA_PHASE_TIMERS): adds
+// seven words after the five work counters.
+#ifdef PA_PHASE_TIMERS
+#define PA_TIMER_BEGIN() unsigned long long t_mark_ = __builtin_readcyclecounter()
+#define PA_TIMER(i)                                                  \
+    do {                                                             \
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); \
+        unsigned long long t_now_ = __builtin_readcyclecounter();    \
+        phase[i] += t_now_ - t_mark_;                                \
+        t_mark_ = t_now_;                                            \
+    } while (0)
+#else
+#define PA_TIMER_BEGIN() do {} while (0)
+#define PA_TIMER(i) do {} while (0)
+#endif
+
+template <int H, int DP8>
 __global__ __launch_bounds__(kWave) void traverse_kernel(TraverseArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int S = (H + kWave - 1) / kWave;
     const int lane = threadIdx.x;
-    const int H = a.H, O = 2 * a.H;
-    const int heap_cells = O > a.sort_n ? O : a.sort_n;
+    const int heap_cells = a.lds_cells;
     float *okey = reinterpret_cast<float *>(smem);
     int *oval = reinterpret_cast<int *>(okey + heap_cells);
+    OpenList<H> open;
+    open.lk = reinterpret_cast<int *>(okey), open.lv = oval;
     int *cand_id = oval + heap_cells;
     float *cand_key = reinterpret_cast<float *>(cand_id + kWave);
     float *qv = cand_key + kWave;
@@ -212,13 +362,17 @@ __global__ __launch_bounds__(kWave) void traverse_kernel(TraverseArgs a) {
         if (q >= a.batch) break;
 
         unsigned long long n_expand = 0, n_adj = 0, n_dist = 0, n_admit = 0;
+#ifdef PA_PHASE_TIMERS
+        unsigned long long phase[7] = {0, 0, 0, 0, 0, 0, 0};
+#endif
+        PA_TIMER_BEGIN();
 
         // fresh visited slice, query to LDS, empty lists
         for (int w = lane * 4; w < a.words_per_slot; w += kWave * 4)
             *reinterpret_cast<uint4 *>(seen + w) = make_uint4(0, 0, 0, 0);
         for (int i = lane; i < dp; i += kWave)
             qv[i] = a.query[(size_t)q * dp + i];
-        for (int i = lane; i < O; i += kWave) okey[i] = INFINITY, oval[i] = -1;
+        open.reset(lane);
         Results<S> res;
         res.init(H, lane);
         __threadfence();
@@ -251,23 +405,37 @@ __global__ __launch_bounds__(kWave) void traverse_kernel(TraverseArgs a) {
                 const int rj = __builtin_amdgcn_readlane(row, j);
                 const float dj =
                     __int_as_float(__builtin_amdgcn_readlane(__float_as_int(d), j));
-                open_replace(okey, oval, O, dj, rj >= 0 ? rj : -2 - (base + j),
-                             lane);
+                open.replace(dj, rj >= 0 ? rj : -2 - (base + j), lane);
             }
         }
 
-        // traverse_cpu.cpp:82-136
+        PA_TIMER(5);
+        // traverse_cpu.cpp:82-136.  The node the next pop will return is the
+        // root of the open list as it stands after the last insert, so its
+        // row of neighbours is requested before the pop and arrives while
+        // the pop's sift runs.
+        auto request_row = [&]() -> int {
+            const int r = OpenList<H>::rl(open.Av, 1);
+            int row = -1;
+            if (r >= 0 && lane < deg) row = a.adj[(size_t)r * deg + lane];
+            return row;
+        };
+        int next_row = request_row();
         for (int step = 0; step < a.max_iter; ++step) {
             float uk;
             int u;
-            open_pop(okey, oval, O, lane, uk, u);
+            open.pop(lane, uk, u);
+            PA_TIMER(0);
             if (u == -1 || uk >= res.worst) break;
             n_expand += 1;
-            if (u < 0) continue;
+            if (u < 0) {
+                next_row = request_row();
+                continue;
+            }
 
-            int v = -1;
-            if (lane < deg) v = a.adj[(size_t)u * deg + lane];
+            const int v = next_row;
             n_adj += deg;
+            PA_TIMER(1);
             bool fresh = false;
             if (v >= 0) {
                 const uint32_t bit = 1u << (v & 31);
@@ -275,12 +443,17 @@ __global__ __launch_bounds__(kWave) void traverse_kernel(TraverseArgs a) {
             }
             const unsigned long long mask = __ballot(fresh);
             const int n = __popcll(mask);
-            if (n == 0) continue;
+            PA_TIMER(2);
+            if (n == 0) {
+                next_row = request_row();
+                continue;
+            }
             if (fresh) cand_id[lane_rank(mask)] = v;
             wave_sync();
             eval_rows<DP8>(a.storage, qv, cand_id, cand_key, n, dp, lane);
             n_dist += n;
             wave_sync();
+            PA_TIMER(3);
 
             // heap_update, traverse_cpu.cpp:25-39, in adjacency order
             const float d = lane < n ? cand_key[lane] : INFINITY;
@@ -294,9 +467,11 @@ __global__ __launch_bounds__(kWave) void traverse_kernel(TraverseArgs a) {
                 if (dj >= res.worst) continue;
                 const int vj = __builtin_amdgcn_readlane(id, j);
                 res.insert(dj, vj, lane);
-                open_replace(okey, oval, O, dj, vj, lane);
+                open.replace(dj, vj, lane);
                 n_admit += 1;
             }
+            next_row = request_row();
+            PA_TIMER(4);
         }
 
         // traverse_cpu.cpp:138-148: storage rows -> global ids, then the
@@ -367,6 +542,10 @@ __global__ __launch_bounds__(kWave) void traverse_kernel(TraverseArgs a) {
             atomicAdd(&a.counters[2], n_dist);
             atomicAdd(&a.counters[3], n_admit);
             atomicAdd(&a.counters[4], (unsigned long long)a.k);
+#ifdef PA_PHASE_TIMERS
+            PA_TIMER(6);
+            for (int i = 0; i < 7; ++i) atomicAdd(&a.counters[5 + i], phase[i]);
+#endif
         }
     }
 }
@@ -452,33 +631,36 @@ int next_pow2(int x) {
 
 typedef void (*TraverseFn)(TraverseArgs);
 
-template <int S>
+template <int H>
 TraverseFn pick_dp(int dp) {
     switch (dp) {
-        case 32: return traverse_kernel<S, 4>;
-        case 64: return traverse_kernel<S, 8>;
-        case 128: return traverse_kernel<S, 16>;
-        default: return traverse_kernel<S, 0>;
+        case 32: return traverse_kernel<H, 4>;
+        case 64: return traverse_kernel<H, 8>;
+        case 128: return traverse_kernel<H, 16>;
+        default: return traverse_kernel<H, 0>;
     }
 }
 
 TraverseFn pick_kernel(int H, int dp) {
-    const int S = (H + kWave - 1) / kWave;
-    switch (S) {
-        case 1: return pick_dp<1>(dp);
-        case 2: return pick_dp<2>(dp);
-        case 3: return pick_dp<3>(dp);
-        case 4: return pick_dp<4>(dp);
-        case 6: return pick_dp<6>(dp);
-        case 8: return pick_dp<8>(dp);
+    switch (H) {
         case 16: return pick_dp<16>(dp);
         case 32: return pick_dp<32>(dp);
+        case 48: return pick_dp<48>(dp);
+        case 64: return pick_dp<64>(dp);
+        case 96: return pick_dp<96>(dp);
+        case 128: return pick_dp<128>(dp);
+        case 192: return pick_dp<192>(dp);
+        case 256: return pick_dp<256>(dp);
+        case 384: return pick_dp<384>(dp);
+        case 512: return pick_dp<512>(dp);
+        case 1024: return pick_dp<1024>(dp);
+        case 2048: return pick_dp<2048>(dp);
         default: return nullptr;
     }
 }
 
 struct Plan {
-    int H, sort_n, lds_bytes, n_slots, words_per_slot;
+    int H, sort_n, lds_cells, lds_bytes, n_slots, words_per_slot;
     size_t workspace_bytes;
     TraverseFn fn;
 };
@@ -490,8 +672,11 @@ int make_plan(int64_t n_storage, int64_t batch, int dp, int ef_total, Plan *p) {
     if (ef_total < 1 || ef_total > PA_MAX_EF_TOTAL) return PA_E_EF;
     p->H = pa_heap_size(ef_total);
     p->sort_n = next_pow2(p->H < kWave ? kWave : p->H);
-    const int cells = 2 * p->H > p->sort_n ? 2 * p->H : p->sort_n;
-    p->lds_bytes = cells * 8 + kWave * 8 + dp * 4;
+    // LDS part of the open list (nodes 256.. of 2H, one spare), reused by the
+    // final sort of sort_n cells
+    const int tail = 2 * p->H + 2 - 256;
+    p->lds_cells = tail > p->sort_n ? tail : p->sort_n;
+    p->lds_bytes = p->lds_cells * 8 + kWave * 8 + dp * 4;
     p->fn = pick_kernel(p->H, dp);
     if (!p->fn) return PA_E_EF;
     int dev = 0, cus = 0, per_cu = 0;
@@ -620,6 +805,7 @@ extern "C" int pa_traverse(int64_t *out_I, float *out_D, const int32_t *adj,
     // traverse_cpu.cpp:18,82
     a.max_iter = 2 * beam * ef < 1024 ? 2 * beam * ef : 1024;
     a.words_per_slot = p.words_per_slot, a.sort_n = p.sort_n;
+    a.lds_cells = p.lds_cells;
 
     hipStream_t stream = (hipStream_t)stream_;
     reset_work_counter<<<1, 1, 0, stream>>>(a.work_counter);
