@@ -1,0 +1,93 @@
+"""Build-time helpers: formats the search path relies on and the properties
+the reference's tests state for them (test/kernel/test_routing.py:6-33,
+test_svd.py, test_graphs.py)."""
+import torch
+
+from pilotann_amd import utils
+
+
+def test_graph_format_and_quality():
+    n, d, deg = 3000, 32, 32
+    x = utils.gaussian_mixture(n, d, 4, 1.0, seed=1)
+    for graph_type in ['nsw', 'nsg']:
+        indptr, indices = utils.graph_init(x, graph_type, deg)
+        assert indptr.dtype == indices.dtype == torch.int64
+        assert indptr.tolist() == [i * deg for i in range(n + 1)]
+        rows = indices.view(n, deg)
+        assert int(rows.max()) < n and int(rows.min()) >= -1
+        assert not (rows == torch.arange(n).unsqueeze(1)).any()      # no self loops
+        # padding only at the end of a row, no repeats inside a row
+        valid = rows >= 0
+        assert (valid[:, :-1] | ~valid[:, 1:]).all()
+        srt = torch.sort(torch.where(valid, rows, -torch.arange(1, deg + 1)), 1).values
+        assert (srt[:, 1:] != srt[:, :-1]).all()
+        # the true nearest neighbour is linked nearly always
+        nn = utils.knn_graph(x, 1)[0]
+        assert (rows == nn).any(1).float().mean() > 0.95
+
+
+def test_sampling_is_seeded_and_closed_under_one_hop():
+    n, deg = 4000, 16
+    x = utils.gaussian_mixture(n, 16, 4, 1.0, seed=2)
+    indptr, indices = utils.graph_init(x, 'nsw', deg)
+    a = utils.graph_sampling(indptr, indices, n // 4, 1, seed=5)
+    b = utils.graph_sampling(indptr, indices, n // 4, 1, seed=5)
+    c = utils.graph_sampling(indptr, indices, n // 4, 1, seed=6)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    assert not torch.equal(a[0], c[0])
+    nodelist, mapping = a
+    assert n // 4 <= nodelist.numel() <= n // 4 + deg + 1
+    assert torch.equal(torch.sort(nodelist).values, nodelist)
+    # the checks of test_traverse_cuda.py:36-40
+    assert int(mapping.max()) + 1 == nodelist.numel()
+    assert (mapping[nodelist] == torch.arange(nodelist.numel())).all()
+    assert int((mapping >= 0).sum()) == nodelist.numel()
+
+
+def test_subgraph_layout():
+    n, deg = 3000, 16
+    x = utils.gaussian_mixture(n, 16, 4, 1.0, seed=3)
+    indptr, indices = utils.graph_init(x, 'nsw', deg)
+    sp, si, nodelist, mapping = utils.subgraph_init(indptr, indices, x, 'nsw',
+                                                    n // 4, deg, seed=1)
+    assert sp.numel() == n + 1 and int(sp[-1]) == si.numel()
+    rowlen = sp[1:] - sp[:-1]
+    assert (rowlen[mapping < 0] == 0).all() and (rowlen[mapping >= 0] == deg).all()
+    assert (mapping[si[si >= 0]] >= 0).all()      # global ids of sampled nodes only
+
+
+def test_router_init_routes_are_nearest_to_their_own_leaves():
+    # test_routing.py:6-33
+    # uniform data as in the reference's fuzz loader (utils/loader.py:31-36)
+    g = torch.Generator().manual_seed(4)
+    x = 2.0 * (torch.rand(40000, 32, generator=g) - 0.5)
+    routes, nodes = utils.router_init(x, None, 32, 32, seed=9)
+    assert routes.shape == (32, 32) and nodes.shape == (32, 32)
+    # rounds draw disjoint node sets: no repeats inside one route's leaves
+    assert all(len(set(r)) == 32 for r in nodes.tolist())
+    dists = torch.cdist(routes.unsqueeze(0).expand(32, -1, -1), x[nodes]).sum(-1)
+    assert torch.equal(torch.argmin(dists, -1), torch.arange(32))
+    again = utils.router_init(x, None, 32, 32, seed=9)
+    assert torch.equal(again[1], nodes)
+    # init_nodes are consumed first (test_routing.py:46-57)
+    init = list(range(100, 132))
+    _, nodes2 = utils.router_init(x, list(init), 8, 32, seed=1)
+    assert set(init) & set(nodes2.flatten().tolist())
+
+
+def test_svd_rotation():
+    # test_svd.py: x V V^T reconstructs x; leading coordinates carry the most
+    x = utils.gaussian_mixture(5000, 48, 8, 1.0, seed=5, decay=0.5)
+    xr, V = utils.svd(x, max_size=10 ** 7)
+    assert torch.allclose(xr @ V.T, x, atol=1e-3)
+    assert torch.allclose(V.T @ V, torch.eye(48), atol=1e-4)
+    energy = xr.square().sum(0)
+    assert (energy[:-1] >= energy[1:] * 0.999).all()
+    xs, Vs = utils.svd(x, max_size=1000, seed=3)      # basis from a sample
+    assert torch.allclose(xs @ Vs.T, x, atol=1e-3)
+
+
+def test_recall():
+    a = torch.tensor([[1, 2, 3], [4, 5, 6]])
+    b = torch.tensor([[3, 2, 9], [7, 8, 9]])
+    assert abs(utils.recall(a, b) - (2 / 3 + 0) / 2) < 1e-9
