@@ -11,6 +11,7 @@ line is printed; `value` is queries per second of that step.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
                     [--n-base N] [--queries B] [--ef EF] [--no-cpu-baseline]
+                    [--copy-calibration]
 """
 import argparse
 import contextlib
@@ -141,6 +142,19 @@ def algorithmic_bytes(counters, B, dp, n_init):
             + C * (w + 4 * dp) + R * (w + 4))
 
 
+def measured_traffic(key):
+    """HBM bytes per launch from the rocprofv3 counter runs summarised under
+    profiles/ (FETCH_SIZE and WRITE_SIZE, each scaled by what a plain copy of
+    known size reads on the same counter), or None for a workload that has
+    not been profiled."""
+    path = os.path.join(ROOT, 'profiles', 'traffic.json')
+    try:
+        with open(path) as f:
+            return json.load(f).get(key, {}).get('hbm_bytes_per_launch')
+    except OSError:
+        return None
+
+
 def cpu_baseline(index, stage, ef, EP_I, EP_D, budget_s=15.0):
     """The host search of the reference (restated in oracle/) on the same
     subgraph, reduced rows and entries, timed on this box's cores on a sample
@@ -185,6 +199,9 @@ def main():
     ap.add_argument('--queries', type=int, default=None)
     ap.add_argument('--ef', type=int, default=None)
     ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--copy-calibration', action='store_true',
+                    help='only run a plain 1 GiB device copy five times (to '
+                         'scale the FETCH_SIZE / WRITE_SIZE counters) and exit')
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get('WORLD_SIZE', '1')) != 1:
         print('bench.py: this build measures one GPU; the search shards by '
@@ -194,6 +211,17 @@ def main():
     if not torch.cuda.is_available():
         print('bench.py: no GPU', file=sys.stderr)
         sys.exit(1)
+
+    if args.copy_calibration:
+        torch.cuda.set_device(0)
+        src = torch.empty(1 << 28, dtype=torch.float32, device='cuda:0').normal_()
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({'copy_calibration': '5 copies of 1 GiB (read 1 GiB, '
+                                              'write 1 GiB each)'}))
+        return
 
     cfg = dict(CONFIGS[args.config])
     if args.n_base:
@@ -266,7 +294,9 @@ def main():
         'roofline': {
             'bound': 'hbm', 'achieved': round(achieved, 1),
             'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
-            'frac': round(achieved / HBM_PEAK_GBS, 4), 'traffic': None,
+            'frac': round(achieved / HBM_PEAK_GBS, 4),
+            'traffic': measured_traffic(
+                f'{args.config}/n={cfg["n"]}/queries={B}/ef={ef}'),
             'kernel': 'traverse_kernel',
             'kernel_ms': round(kernel_ms, 4),
             'algorithmic_bytes_per_launch': launch_bytes,
