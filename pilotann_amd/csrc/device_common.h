@@ -49,6 +49,29 @@ __device__ __forceinline__ float wave_max(float x) {
 }
 
 
+// Maximum of a signed integer over the wavefront, in every lane: six DPP
+// steps (rows of 16 by quad_perm and mirrors, then row_bcast15 / row_bcast31
+// into the upper rows) and a read of lane 63.  Written as v_max_i32_dpp so
+// that each step is one instruction; the s_nop covers the two wait states a
+// DPP read needs after a vector write of the same register.
+__device__ __forceinline__ int wave_max_key(int x) {
+    asm("s_nop 1\n\t"
+        "v_max_i32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_i32_dpp %0, %0, %0 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_i32_dpp %0, %0, %0 row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_i32_dpp %0, %0, %0 row_mirror row_mask:0xf bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_i32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+        "s_nop 1\n\t"
+        "v_max_i32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+        "s_nop 1"
+        : "+v"(x));
+    return __builtin_amdgcn_readlane(x, kWave - 1);
+}
+
 // Squared L2 between a query held in LDS and one storage row, in the order of
 // the reference's host code (extension/inc/distance.h:31-55): element j of
 // every group of eight goes to accumulator j with one FMA, the eight

@@ -34,6 +34,7 @@ namespace {
 
 constexpr int kSlotAlignWords = 256;   // bitmask slice: multiple of 1 KiB
 constexpr int kWorkCounterBytes = 256; // head of the workspace
+constexpr int kSeenCache = 1024;       // LDS cells remembering visited rows
 
 // ---- open list: heapq.cuh, top of the heap in registers ----------------------
 //
@@ -151,39 +152,37 @@ struct OpenList {
     }
 
     // heapq.cuh:37-45 with the sift of :13-29: the root leaves, (inf, -1)
-    // sinks along the smaller child (left on ties) while that child is finite.
-    // Levels 1..kDepth-1 are complete; on level kDepth only nodes up to kSize
-    // exist, and node kSize has no sibling.
-    __device__ __forceinline__ void pop(int lane, float &out_k, int &out_v) {
-        out_k = key_to_float(rl(Ak, 1));
+    // sinks along the smaller child (left on ties).  The reference stops when
+    // that child is (inf, -1) too; going on to the bottom instead only copies
+    // (inf, -1) over (inf, -1) — every infinite cell carries -1 — so the
+    // final state is the same and the walk is straight-line code.  Levels
+    // 1..kDepth-1 are complete; on level kDepth only nodes up to kSize exist
+    // and node kSize has no sibling.
+    __device__ __forceinline__ void pop(int lane, int &out_k, int &out_v) {
+        out_k = rl(Ak, 1);
         out_v = rl(Av, 1);
         int j = 1;
 #pragma unroll
-        for (int L = 1; L <= kDepth; ++L) {
+        for (int L = 1; L < kDepth; ++L) {
             const int c = 2 * j;
             int ka, kb, va, vb;
-            if (L == kDepth) {
-                if (c > kSize) break;
-                pair(kind(L), true, c, ka, kb, va, vb);
-                kb = c == kSize ? ka : kb;
-            } else {
-                pair(kind(L), true, c, ka, kb, va, vb);
-            }
+            pair(kind(L), true, c, ka, kb, va, vb);
             const int ck = min(ka, kb);
-            if (ck >= kInf) {
-                put(kind(L - 1), j, kInf, -1, lane);
-                wave_sync();
-                return;
-            }
             put(kind(L - 1), j, ck, ck != ka ? vb : va, lane);
             j = add_if_ne(c, ck, ka);
-            if (L == kDepth) {
-                put(kind(L), j, kInf, -1, lane);
-                wave_sync();
-                return;
-            }
         }
-        put(kind(kDepth - 1), j, kInf, -1, lane);
+        const int c = 2 * j;
+        if (c <= kSize) {
+            int ka, kb, va, vb;
+            pair(kind(kDepth), true, c, ka, kb, va, vb);
+            kb = c == kSize ? ka : kb;
+            const int ck = min(ka, kb);
+            put(kind(kDepth - 1), j, ck, ck != ka ? vb : va, lane);
+            j = add_if_ne(c, ck, ka);
+            put(kind(kDepth), j, kInf, -1, lane);
+        } else {
+            put(kind(kDepth - 1), j, kInf, -1, lane);
+        }
         wave_sync();
     }
 
@@ -191,8 +190,7 @@ struct OpenList {
     // ties), overwrite it when the new key is strictly smaller, let the new
     // entry rise.  The walk keeps the keys it passes, so the rise needs no
     // further key reads.
-    __device__ __forceinline__ void replace(float key, int v, int lane) {
-        const int k = float_to_key(key);
+    __device__ __forceinline__ void replace(int k, int v, int lane) {
         int pj[kDepth + 1], pk[kDepth + 1];
         pj[0] = 1, pk[0] = rl(Ak, 1);
         int deepest = kDepth;
@@ -241,40 +239,41 @@ struct OpenList {
 
 template <int S>
 struct Results {
-    float key[S];
+    static constexpr int kInf = 0x7f800000;      // float_to_key(+inf)
+    static constexpr int kNegInf = (int)0x807fffff;  // float_to_key(-inf)
+    int key[S];   // float_to_key of the distance
     int val[S];
-    float lane_max;
-    float worst;  // uniform
+    int lane_max;
+    int worst;    // uniform
 
     __device__ __forceinline__ void init(int H, int lane) {
-        lane_max = -INFINITY;
+        lane_max = kNegInf;
 #pragma unroll
         for (int s = 0; s < S; ++s) {
-            key[s] = (s * kWave + lane < H) ? INFINITY : -INFINITY;
+            key[s] = (s * kWave + lane < H) ? kInf : kNegInf;
             val[s] = -1;
-            lane_max = fmaxf(lane_max, key[s]);
+            lane_max = max(lane_max, key[s]);
         }
-        worst = INFINITY;
+        worst = kInf;
     }
-    // Caller has checked !(d >= worst).
-    __device__ __forceinline__ void insert(float d, int v, int lane) {
-        unsigned long long holders = __ballot(lane_max == worst);
-        int owner = __builtin_ctzll(holders);
-        if (lane == owner) {
-            bool done = false;
-            float m = -INFINITY;
+    // Caller has checked k < worst.  The first lane whose maximum is the
+    // worst replaces its first cell that holds it (branch-free: every lane
+    // runs the same selects).
+    __device__ __forceinline__ void insert(int k, int v, int lane) {
+        const unsigned long long holders = __ballot(lane_max == worst);
+        const bool mine = lane == __builtin_ctzll(holders);
+        bool open = mine;
+        int m = kNegInf;
 #pragma unroll
-            for (int s = 0; s < S; ++s) {
-                if (!done && key[s] == worst) {
-                    key[s] = d;
-                    val[s] = v;
-                    done = true;
-                }
-                m = fmaxf(m, key[s]);
-            }
-            lane_max = m;
+        for (int s = 0; s < S; ++s) {
+            const bool hit = open && key[s] == worst;
+            key[s] = hit ? k : key[s];
+            val[s] = hit ? v : val[s];
+            open = open && !hit;
+            m = max(m, key[s]);
         }
-        worst = wave_max(lane_max);
+        lane_max = m;
+        worst = wave_max_key(lane_max);
     }
 };
 
@@ -338,8 +337,15 @@ __global__ void reset_work_counter(int *counter) { *counter = 0; }
 #define PA_TIMER(i) do {} while (0)
 #endif
 
+// Tuning builds may pin the register budget (-DPA_WAVES_PER_EU=n).
+#ifdef PA_WAVES_PER_EU
+#define PA_OCCUPANCY __attribute__((amdgpu_waves_per_eu(PA_WAVES_PER_EU, PA_WAVES_PER_EU)))
+#else
+#define PA_OCCUPANCY
+#endif
+
 template <int H, int DP8>
-__global__ __launch_bounds__(kWave) void traverse_kernel(TraverseArgs a) {
+__global__ __launch_bounds__(kWave) PA_OCCUPANCY void traverse_kernel(TraverseArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int S = (H + kWave - 1) / kWave;
     const int lane = threadIdx.x;
@@ -352,6 +358,7 @@ __global__ __launch_bounds__(kWave) void traverse_kernel(TraverseArgs a) {
     float *cand_key = reinterpret_cast<float *>(cand_id + kWave);
     float *qv = cand_key + kWave;
     const int dp = DP8 ? DP8 * 8 : a.dp;
+    int *seen_cache = reinterpret_cast<int *>(qv + dp);
     const int deg = a.deg;
     uint32_t *seen = a.seen + (size_t)blockIdx.x * (size_t)a.words_per_slot;
 
@@ -372,6 +379,7 @@ __global__ __launch_bounds__(kWave) void traverse_kernel(TraverseArgs a) {
             *reinterpret_cast<uint4 *>(seen + w) = make_uint4(0, 0, 0, 0);
         for (int i = lane; i < dp; i += kWave)
             qv[i] = a.query[(size_t)q * dp + i];
+        for (int i = lane; i < kSeenCache; i += kWave) seen_cache[i] = -1;
         open.reset(lane);
         Results<S> res;
         res.init(H, lane);
@@ -405,73 +413,98 @@ __global__ __launch_bounds__(kWave) void traverse_kernel(TraverseArgs a) {
                 const int rj = __builtin_amdgcn_readlane(row, j);
                 const float dj =
                     __int_as_float(__builtin_amdgcn_readlane(__float_as_int(d), j));
-                open.replace(dj, rj >= 0 ? rj : -2 - (base + j), lane);
+                open.replace(float_to_key(dj), rj >= 0 ? rj : -2 - (base + j), lane);
             }
         }
 
         PA_TIMER(5);
-        // traverse_cpu.cpp:82-136.  The node the next pop will return is the
-        // root of the open list as it stands after the last insert, so its
-        // row of neighbours is requested before the pop and arrives while
-        // the pop's sift runs.
-        auto request_row = [&]() -> int {
-            const int r = OpenList<H>::rl(open.Av, 1);
+        // traverse_cpu.cpp:82-136, software-pipelined.  The node a pop will
+        // return is the root of the open list as it stands after the last
+        // insert, so once a step's inserts are done the next step's node is
+        // certain: its neighbours' visited bits are tested and set *before*
+        // the pop (the atomics are in flight while the pop sifts).  Its row of
+        // neighbour ids is needed for that, and is requested even earlier,
+        // before the inserts, for the node that will most likely be the root
+        // after them: the best new candidate if it beats the present root and
+        // the admission bound, else the present root.  That load is only a
+        // read; when the guess is wrong the row is loaded again.  If the
+        // search ends at the next pop instead, the marks set for a node that
+        // is never expanded are harmless: the slice is cleared per query.
+        auto load_row = [&](int r) -> int {
             int row = -1;
             if (r >= 0 && lane < deg) row = a.adj[(size_t)r * deg + lane];
             return row;
         };
-        int next_row = request_row();
+        // Returns the bitmask word before the OR; it is looked at only after
+        // the pop.  Most neighbours of a node were seen a few steps ago: a
+        // direct-mapped LDS table of rows whose bit is known to be set
+        // answers for them without going to memory.  A row enters the table
+        // only after its atomic has been issued, so a hit is always right; a
+        // miss (never seen, or displaced) asks the bitmask, which is exact.
+        auto test_and_set = [&](int v) -> uint32_t {
+            uint32_t before = 0xffffffffu;
+            if (v >= 0) {
+                const int cell = ((uint32_t)v * 2654435761u) >> 22;
+                if (seen_cache[cell] != v) {
+                    before = atomicOr(&seen[v >> 5], 1u << (v & 31));
+                    seen_cache[cell] = v;
+                }
+            }
+            return before;
+        };
+        int v = load_row(OpenList<H>::rl(open.Av, 1));
+        uint32_t before = test_and_set(v);
         for (int step = 0; step < a.max_iter; ++step) {
-            float uk;
-            int u;
+            int uk, u;
             open.pop(lane, uk, u);
             PA_TIMER(0);
             if (u == -1 || uk >= res.worst) break;
             n_expand += 1;
-            if (u < 0) {
-                next_row = request_row();
-                continue;
-            }
+            int guess = -3, guess_row = -1;
+            if (u >= 0) {
+                n_adj += deg;
+                const bool fresh = !((before >> (v & 31)) & 1u);
+                const unsigned long long mask = __ballot(fresh);
+                const int n = __popcll(mask);
+                PA_TIMER(2);
+                if (n > 0) {
+                    if (fresh) cand_id[lane_rank(mask)] = v;
+                    wave_sync();
+                    eval_rows<DP8>(a.storage, qv, cand_id, cand_key, n, dp, lane);
+                    n_dist += n;
+                    wave_sync();
+                    PA_TIMER(3);
 
-            const int v = next_row;
-            n_adj += deg;
+                    const int d = float_to_key(lane < n ? cand_key[lane] : INFINITY);
+                    const int id = lane < n ? cand_id[lane] : -1;
+                    // most likely next node; first candidate on ties, as the
+                    // rise of an equal key stops below the older one
+                    const int d_min = -wave_max_key(-d);
+                    guess = OpenList<H>::rl(open.Av, 1);
+                    if (d_min < OpenList<H>::rl(open.Ak, 1) && d_min < res.worst)
+                        guess = __builtin_amdgcn_readlane(
+                            id, __builtin_ctzll(__ballot(d == d_min)));
+                    guess_row = load_row(guess);
+
+                    // heap_update, traverse_cpu.cpp:25-39, in adjacency order
+                    unsigned long long todo = __ballot(d < res.worst);
+                    while (todo) {
+                        const int j = __builtin_ctzll(todo);
+                        todo &= todo - 1;
+                        const int dj = __builtin_amdgcn_readlane(d, j);
+                        if (dj >= res.worst) continue;
+                        const int vj = __builtin_amdgcn_readlane(id, j);
+                        res.insert(dj, vj, lane);
+                        open.replace(dj, vj, lane);
+                        n_admit += 1;
+                    }
+                    PA_TIMER(4);
+                }
+            }
+            const int r = OpenList<H>::rl(open.Av, 1);
+            v = r == guess ? guess_row : load_row(r);
+            before = test_and_set(v);
             PA_TIMER(1);
-            bool fresh = false;
-            if (v >= 0) {
-                const uint32_t bit = 1u << (v & 31);
-                fresh = !(atomicOr(&seen[v >> 5], bit) & bit);
-            }
-            const unsigned long long mask = __ballot(fresh);
-            const int n = __popcll(mask);
-            PA_TIMER(2);
-            if (n == 0) {
-                next_row = request_row();
-                continue;
-            }
-            if (fresh) cand_id[lane_rank(mask)] = v;
-            wave_sync();
-            eval_rows<DP8>(a.storage, qv, cand_id, cand_key, n, dp, lane);
-            n_dist += n;
-            wave_sync();
-            PA_TIMER(3);
-
-            // heap_update, traverse_cpu.cpp:25-39, in adjacency order
-            const float d = lane < n ? cand_key[lane] : INFINITY;
-            const int id = lane < n ? cand_id[lane] : -1;
-            unsigned long long todo = __ballot(!(d >= res.worst));
-            while (todo) {
-                const int j = __builtin_ctzll(todo);
-                todo &= todo - 1;
-                const float dj =
-                    __int_as_float(__builtin_amdgcn_readlane(__float_as_int(d), j));
-                if (dj >= res.worst) continue;
-                const int vj = __builtin_amdgcn_readlane(id, j);
-                res.insert(dj, vj, lane);
-                open.replace(dj, vj, lane);
-                n_admit += 1;
-            }
-            next_row = request_row();
-            PA_TIMER(4);
         }
 
         // traverse_cpu.cpp:138-148: storage rows -> global ids, then the
@@ -488,12 +521,12 @@ __global__ __launch_bounds__(kWave) void traverse_kernel(TraverseArgs a) {
                 d = eD[i];
                 if (g >= 0 && g < a.n_nodes) u = (int)g;
             }
-            unsigned long long todo = __ballot(u >= 0 && !(d >= res.worst));
+            const int dk = float_to_key(d);
+            unsigned long long todo = __ballot(u >= 0 && dk < res.worst);
             while (todo) {
                 const int j = __builtin_ctzll(todo);
                 todo &= todo - 1;
-                const float dj =
-                    __int_as_float(__builtin_amdgcn_readlane(__float_as_int(d), j));
+                const int dj = __builtin_amdgcn_readlane(dk, j);
                 if (dj >= res.worst) continue;
                 res.insert(dj, __builtin_amdgcn_readlane(u, j), lane);
             }
@@ -508,7 +541,7 @@ __global__ __launch_bounds__(kWave) void traverse_kernel(TraverseArgs a) {
 #pragma unroll
         for (int s = 0; s < S; ++s) {
             const int e = s * kWave + lane;
-            if (e < H) okey[e] = res.key[s], oval[e] = res.val[s];
+            if (e < H) okey[e] = key_to_float(res.key[s]), oval[e] = res.val[s];
         }
         wave_sync();
         for (int size = 2; size <= a.sort_n; size <<= 1) {
@@ -676,7 +709,10 @@ int make_plan(int64_t n_storage, int64_t batch, int dp, int ef_total, Plan *p) {
     // final sort of sort_n cells
     const int tail = 2 * p->H + 2 - 256;
     p->lds_cells = tail > p->sort_n ? tail : p->sort_n;
-    p->lds_bytes = p->lds_cells * 8 + kWave * 8 + dp * 4;
+    p->lds_bytes = p->lds_cells * 8 + kWave * 8 + dp * 4 + kSeenCache * 4;
+#ifdef PA_EXTRA_LDS  // tuning builds: lower the residency without touching code
+    p->lds_bytes += PA_EXTRA_LDS;
+#endif
     p->fn = pick_kernel(p->H, dp);
     if (!p->fn) return PA_E_EF;
     int dev = 0, cus = 0, per_cu = 0;
@@ -688,8 +724,15 @@ int make_plan(int64_t n_storage, int64_t batch, int dp, int ef_total, Plan *p) {
             &per_cu, reinterpret_cast<const void *>(p->fn), kWave, p->lds_bytes);
     if (e != hipSuccess) return (int)e;
     if (per_cu < 1) per_cu = 1;
+    // as many wavefronts as stay resident, but no more than give every one
+    // the same number of queries: a last round that fills a fraction of the
+    // GPU costs a whole query time
     int64_t slots = (int64_t)per_cu * cus;
-    if (slots > batch) slots = batch;
+    if (slots < 1) slots = 1;
+    if (batch > 0) {
+        const int64_t rounds = (batch + slots - 1) / slots;
+        slots = (batch + rounds - 1) / rounds;
+    }
     if (slots < 1) slots = 1;
     p->n_slots = (int)slots;
     p->words_per_slot = round_up((n_storage + 31) / 32, kSlotAlignWords);
