@@ -34,7 +34,8 @@ namespace {
 
 constexpr int kSlotAlignWords = 256;   // bitmask slice: multiple of 1 KiB
 constexpr int kWorkCounterBytes = 256; // head of the workspace
-constexpr int kSeenCache = 1024;       // LDS cells remembering visited rows
+constexpr int kSeenCacheLog2 = 10;
+constexpr int kSeenCache = 1 << kSeenCacheLog2;  // LDS words remembering visited rows
 
 // ---- open list: heapq.cuh, top of the heap in registers ----------------------
 //
@@ -122,6 +123,15 @@ struct OpenList {
             ka = uni(k2.x), kb = uni(k2.y);
         }
     }
+    __device__ __forceinline__ int key_of(const int KIND, int j) const {
+        if (KIND == 0) return rl(Ak, j);
+        if (KIND == 1) return rl(Bk, j - 64);
+        if (KIND == 2) {
+            const int l = (j - 128) >> 1;
+            return (j & 1) ? rl(Dk, l) : rl(Ck, l);
+        }
+        return uni(lk[j - kRegNodes]);
+    }
     __device__ __forceinline__ int val_of(const int KIND, int j) const {
         if (KIND == 0) return rl(Av, j);
         if (KIND == 1) return rl(Bv, j - 64);
@@ -188,40 +198,53 @@ struct OpenList {
 
     // heapq.cuh:47-77: walk to a leaf through the larger child (left on
     // ties), overwrite it when the new key is strictly smaller, let the new
-    // entry rise.  The walk keeps the keys it passes, so the rise needs no
-    // further key reads.
+    // entry rise.
     __device__ __forceinline__ void replace(int k, int v, int lane) {
-        int pj[kDepth + 1], pk[kDepth + 1];
-        pj[0] = 1, pk[0] = rl(Ak, 1);
-        int deepest = kDepth;
+        int j = 1;
+        int leaf = rl(Ak, 1);
 #pragma unroll
-        for (int L = 1; L <= kDepth; ++L) {
-            const int c = 2 * pj[L - 1];
+        for (int L = 1; L < kDepth; ++L) {
+            const int c = 2 * j;
             int ka, kb, va, vb;
-            if (L == kDepth) {
-                if (c > kSize) {
-                    deepest = kDepth - 1;
-                    pj[L] = 0, pk[L] = 0;
-                    break;
-                }
-                pair(kind(L), false, c, ka, kb, va, vb);
-                kb = c == kSize ? ka : kb;
-            } else {
-                pair(kind(L), false, c, ka, kb, va, vb);
-            }
-            pk[L] = max(ka, kb);
-            pj[L] = add_if_ne(c, pk[L], ka);
+            pair(kind(L), false, c, ka, kb, va, vb);
+            leaf = max(ka, kb);
+            j = add_if_ne(c, leaf, ka);
         }
-        if (k >= (deepest == kDepth ? pk[kDepth] : pk[kDepth - 1])) return;
-#pragma unroll
-        for (int L = kDepth; L >= 1; --L) {
-            if (L == kDepth && deepest != kDepth) continue;
-            if (pk[L - 1] <= k) {
-                put(kind(L), pj[L], k, v, lane);
+        bool bottom = false;  // the walk reached level kDepth
+        {
+            const int c = 2 * j;
+            if (c <= kSize) {
+                int ka, kb, va, vb;
+                pair(kind(kDepth), false, c, ka, kb, va, vb);
+                kb = c == kSize ? ka : kb;
+                leaf = max(ka, kb);
+                j = add_if_ne(c, leaf, ka);
+                bottom = true;
+            }
+        }
+        if (k >= leaf) return;
+        if (bottom) {
+            const int up = j >> 1;
+            const int pk = key_of(kind(kDepth - 1), up);
+            if (pk <= k) {
+                put(kind(kDepth), j, k, v, lane);
                 wave_sync();
                 return;
             }
-            put(kind(L), pj[L], pk[L - 1], val_of(kind(L - 1), pj[L - 1]), lane);
+            put(kind(kDepth), j, pk, val_of(kind(kDepth - 1), up), lane);
+            j = up;
+        }
+#pragma unroll
+        for (int L = kDepth - 1; L >= 1; --L) {
+            const int up = j >> 1;
+            const int pk = key_of(kind(L - 1), up);
+            if (pk <= k) {
+                put(kind(L), j, k, v, lane);
+                wave_sync();
+                return;
+            }
+            put(kind(L), j, pk, val_of(kind(L - 1), up), lane);
+            j = up;
         }
         put(0, 1, k, v, lane);
         wave_sync();
@@ -337,15 +360,17 @@ __global__ void reset_work_counter(int *counter) { *counter = 0; }
 #define PA_TIMER(i) do {} while (0)
 #endif
 
-// Tuning builds may pin the register budget (-DPA_WAVES_PER_EU=n).
+// Up to H = 256 the kernel fits the register budget of five wavefronts per
+// SIMD (96 VGPRs), which measures faster than four; larger result lists need
+// more registers and are left to the compiler.
 #ifdef PA_WAVES_PER_EU
-#define PA_OCCUPANCY __attribute__((amdgpu_waves_per_eu(PA_WAVES_PER_EU, PA_WAVES_PER_EU)))
+#define PA_OCCUPANCY(H) __attribute__((amdgpu_waves_per_eu(PA_WAVES_PER_EU, PA_WAVES_PER_EU)))
 #else
-#define PA_OCCUPANCY
+#define PA_OCCUPANCY(H) __attribute__((amdgpu_waves_per_eu((H) <= 256 ? 5 : 1, (H) <= 256 ? 5 : 8)))
 #endif
 
 template <int H, int DP8>
-__global__ __launch_bounds__(kWave) PA_OCCUPANCY void traverse_kernel(TraverseArgs a) {
+__global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(TraverseArgs a) {
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int S = (H + kWave - 1) / kWave;
     const int lane = threadIdx.x;
@@ -358,7 +383,8 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY void traverse_kernel(TraverseAr
     float *cand_key = reinterpret_cast<float *>(cand_id + kWave);
     float *qv = cand_key + kWave;
     const int dp = DP8 ? DP8 * 8 : a.dp;
-    int *seen_cache = reinterpret_cast<int *>(qv + dp);
+    uint32_t *seen_cache = reinterpret_cast<uint32_t *>(qv + dp);
+    const bool use_cache = a.n_storage <= (0xffff << kSeenCacheLog2);
     const int deg = a.deg;
     uint32_t *seen = a.seen + (size_t)blockIdx.x * (size_t)a.words_per_slot;
 
@@ -368,7 +394,7 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY void traverse_kernel(TraverseAr
         q = uni(q);
         if (q >= a.batch) break;
 
-        unsigned long long n_expand = 0, n_adj = 0, n_dist = 0, n_admit = 0;
+        unsigned n_expand = 0, n_adj = 0, n_dist = 0, n_admit = 0;
 #ifdef PA_PHASE_TIMERS
         unsigned long long phase[7] = {0, 0, 0, 0, 0, 0, 0};
 #endif
@@ -379,7 +405,7 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY void traverse_kernel(TraverseAr
             *reinterpret_cast<uint4 *>(seen + w) = make_uint4(0, 0, 0, 0);
         for (int i = lane; i < dp; i += kWave)
             qv[i] = a.query[(size_t)q * dp + i];
-        for (int i = lane; i < kSeenCache; i += kWave) seen_cache[i] = -1;
+        for (int i = lane; i < kSeenCache; i += kWave) seen_cache[i] = 0xffffffffu;
         open.reset(lane);
         Results<S> res;
         res.init(H, lane);
@@ -437,17 +463,21 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY void traverse_kernel(TraverseAr
         };
         // Returns the bitmask word before the OR; it is looked at only after
         // the pop.  Most neighbours of a node were seen a few steps ago: a
-        // direct-mapped LDS table of rows whose bit is known to be set
-        // answers for them without going to memory.  A row enters the table
-        // only after its atomic has been issued, so a hit is always right; a
-        // miss (never seen, or displaced) asks the bitmask, which is exact.
+        // two-way LDS table of rows whose bit is known to be set answers for
+        // them without going to memory.  Word r mod 1024 holds the 16-bit
+        // tags r / 1024 of the two rows seen last (newest in the low half).
+        // A row enters the table only after its atomic has been issued, so a
+        // hit is always right; a miss (never seen, or displaced) asks the
+        // bitmask, which is exact.
         auto test_and_set = [&](int v) -> uint32_t {
             uint32_t before = 0xffffffffu;
             if (v >= 0) {
-                const int cell = ((uint32_t)v * 2654435761u) >> 22;
-                if (seen_cache[cell] != v) {
+                const int cell = v & (kSeenCache - 1);
+                const uint32_t tag = (uint32_t)v >> kSeenCacheLog2;
+                const uint32_t ways = use_cache ? seen_cache[cell] : 0xffffffffu;
+                if ((ways & 0xffffu) != tag && (ways >> 16) != tag) {
                     before = atomicOr(&seen[v >> 5], 1u << (v & 31));
-                    seen_cache[cell] = v;
+                    if (use_cache) seen_cache[cell] = (ways << 16) | tag;
                 }
             }
             return before;
@@ -570,10 +600,10 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY void traverse_kernel(TraverseAr
         wave_sync();
 
         if (a.counters && lane == 0) {
-            atomicAdd(&a.counters[0], n_expand);
-            atomicAdd(&a.counters[1], n_adj);
-            atomicAdd(&a.counters[2], n_dist);
-            atomicAdd(&a.counters[3], n_admit);
+            atomicAdd(&a.counters[0], (unsigned long long)n_expand);
+            atomicAdd(&a.counters[1], (unsigned long long)n_adj);
+            atomicAdd(&a.counters[2], (unsigned long long)n_dist);
+            atomicAdd(&a.counters[3], (unsigned long long)n_admit);
             atomicAdd(&a.counters[4], (unsigned long long)a.k);
 #ifdef PA_PHASE_TIMERS
             PA_TIMER(6);
@@ -724,15 +754,9 @@ int make_plan(int64_t n_storage, int64_t batch, int dp, int ef_total, Plan *p) {
             &per_cu, reinterpret_cast<const void *>(p->fn), kWave, p->lds_bytes);
     if (e != hipSuccess) return (int)e;
     if (per_cu < 1) per_cu = 1;
-    // as many wavefronts as stay resident, but no more than give every one
-    // the same number of queries: a last round that fills a fraction of the
-    // GPU costs a whole query time
     int64_t slots = (int64_t)per_cu * cus;
     if (slots < 1) slots = 1;
-    if (batch > 0) {
-        const int64_t rounds = (batch + slots - 1) / slots;
-        slots = (batch + rounds - 1) / rounds;
-    }
+    if (slots > batch) slots = batch;
     if (slots < 1) slots = 1;
     p->n_slots = (int)slots;
     p->words_per_slot = round_up((n_storage + 31) / 32, kSlotAlignWords);
