@@ -73,6 +73,16 @@ __device__ __forceinline__ int add_if_ne(int c, int a, int b) {
 
 constexpr int floor_log2(int x) { return x <= 1 ? 0 : 1 + floor_log2(x >> 1); }
 
+// c + bit `idx` of a 64-bit lane mask, on the scalar unit.
+__device__ __forceinline__ int add_if_bit(int c, unsigned long long mask, int idx) {
+    int r;
+    asm("s_bitcmp1_b64 %1, %2\n\ts_addc_u32 %0, %3, 0"
+        : "=s"(r)
+        : "s"(mask), "s"(idx), "s"(c)
+        : "scc");
+    return r;
+}
+
 template <int H>
 struct OpenList {
     static constexpr int kSize = 2 * H;           // cells of the reference heap
@@ -161,38 +171,76 @@ struct OpenList {
         }
     }
 
+    // Which child a walk takes, for every sibling pair of the register levels
+    // at once: lane-parallel compares against the sibling (one DPP move per
+    // bank), read back as lane masks, so that a level of the walk is three
+    // scalar instructions and no register read.  LARGER selects the rule of
+    // heap_replace (strictly larger right child), else that of the sift of a
+    // pop (strictly smaller right child); left wins ties in both.  In banks A
+    // and B bit i of the mask tells about the pair whose right child sits in
+    // lane i; in banks C/D lane i holds both children.
+    struct Choice {
+        unsigned long long a, b, cd;
+    };
+    template <bool LARGER>
+    __device__ __forceinline__ Choice choices() const {
+        Choice ch;
+        const int sa = __builtin_amdgcn_update_dpp(Ak, Ak, 0xB1, 0xF, 0xF, false);
+        ch.a = __ballot(LARGER ? Ak > sa : Ak < sa);
+        ch.b = 0, ch.cd = 0;
+        if (kDepth >= 6) {
+            const int sb = __builtin_amdgcn_update_dpp(Bk, Bk, 0xB1, 0xF, 0xF, false);
+            ch.b = __ballot(LARGER ? Bk > sb : Bk < sb);
+        }
+        if (kDepth >= 7) ch.cd = __ballot(LARGER ? Dk > Ck : Dk < Ck);
+        return ch;
+    }
+    // the child of j the walk takes on register level L (1..7), L < kDepth
+    // or the pair is known to be complete
+    __device__ __forceinline__ int step_down(const int L, int j,
+                                             const Choice &ch) const {
+        const int c = 2 * j;
+        if (kind(L) == 0) return add_if_bit(c, ch.a, c + 1);
+        if (kind(L) == 1) return add_if_bit(c, ch.b, c + 1 - 64);
+        return add_if_bit(c, ch.cd, j - 64);
+    }
+
     // heapq.cuh:37-45 with the sift of :13-29: the root leaves, (inf, -1)
     // sinks along the smaller child (left on ties).  The reference stops when
     // that child is (inf, -1) too; going on to the bottom instead only copies
     // (inf, -1) over (inf, -1) — every infinite cell carries -1 — so the
     // final state is the same and the walk is straight-line code.  Levels
     // 1..kDepth-1 are complete; on level kDepth only nodes up to kSize exist
-    // and node kSize has no sibling.
+    // and node kSize has no sibling (its absent sibling's cell holds +inf and
+    // is never the smaller one).
     __device__ __forceinline__ void pop(int lane, int &out_k, int &out_v) {
         out_k = rl(Ak, 1);
         out_v = rl(Av, 1);
+        const Choice ch = choices<false>();
         int j = 1;
 #pragma unroll
-        for (int L = 1; L < kDepth; ++L) {
-            const int c = 2 * j;
-            int ka, kb, va, vb;
-            pair(kind(L), true, c, ka, kb, va, vb);
-            const int ck = min(ka, kb);
-            put(kind(L - 1), j, ck, ck != ka ? vb : va, lane);
-            j = add_if_ne(c, ck, ka);
+        for (int L = 1; L <= kDepth; ++L) {
+            if (L == kDepth && 2 * j > kSize) {
+                put(kind(L - 1), j, kInf, -1, lane);
+                wave_sync();
+                return;
+            }
+            int c, ck, cv;
+            if (kind(L) <= 2) {
+                c = step_down(L, j, ch);
+                ck = key_of(kind(L), c), cv = val_of(kind(L), c);
+            } else {
+                int ka, kb, va, vb;
+                pair(3, true, 2 * j, ka, kb, va, vb);
+                if (L == kDepth) kb = 2 * j == kSize ? ka : kb;
+                ck = min(ka, kb);
+                cv = ck != ka ? vb : va;
+                c = add_if_ne(2 * j, ck, ka);
+            }
+            put(kind(L - 1), j, ck, cv, lane);
+            j = c;
         }
-        const int c = 2 * j;
-        if (c <= kSize) {
-            int ka, kb, va, vb;
-            pair(kind(kDepth), true, c, ka, kb, va, vb);
-            kb = c == kSize ? ka : kb;
-            const int ck = min(ka, kb);
-            put(kind(kDepth - 1), j, ck, ck != ka ? vb : va, lane);
-            j = add_if_ne(c, ck, ka);
-            put(kind(kDepth), j, kInf, -1, lane);
-        } else {
-            put(kind(kDepth - 1), j, kInf, -1, lane);
-        }
+        put(kind(kDepth), j, kInf, -1, lane);
         wave_sync();
     }
 
@@ -200,29 +248,27 @@ struct OpenList {
     // ties), overwrite it when the new key is strictly smaller, let the new
     // entry rise.
     __device__ __forceinline__ void replace(int k, int v, int lane) {
+        const Choice ch = choices<true>();
         int j = 1;
-        int leaf = rl(Ak, 1);
+        bool bottom = true;  // the walk reached level kDepth
 #pragma unroll
-        for (int L = 1; L < kDepth; ++L) {
-            const int c = 2 * j;
-            int ka, kb, va, vb;
-            pair(kind(L), false, c, ka, kb, va, vb);
-            leaf = max(ka, kb);
-            j = add_if_ne(c, leaf, ka);
-        }
-        bool bottom = false;  // the walk reached level kDepth
-        {
-            const int c = 2 * j;
-            if (c <= kSize) {
+        for (int L = 1; L <= kDepth; ++L) {
+            if (L == kDepth && 2 * j > kSize) {
+                bottom = false;
+                break;
+            }
+            if (kind(L) <= 2) {
+                // node kSize has no sibling: the left child it is
+                j = (L == kDepth && 2 * j == kSize) ? 2 * j : step_down(L, j, ch);
+            } else {
                 int ka, kb, va, vb;
-                pair(kind(kDepth), false, c, ka, kb, va, vb);
-                kb = c == kSize ? ka : kb;
-                leaf = max(ka, kb);
-                j = add_if_ne(c, leaf, ka);
-                bottom = true;
+                pair(3, false, 2 * j, ka, kb, va, vb);
+                if (L == kDepth) kb = 2 * j == kSize ? ka : kb;
+                j = add_if_ne(2 * j, max(ka, kb), ka);
             }
         }
-        if (k >= leaf) return;
+        if (k >= (bottom ? key_of(kind(kDepth), j) : key_of(kind(kDepth - 1), j)))
+            return;
         if (bottom) {
             const int up = j >> 1;
             const int pk = key_of(kind(kDepth - 1), up);
