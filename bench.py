@@ -289,7 +289,8 @@ def main():
         'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
         'dtype': 'f32', 'data': 'synthetic',
         'config': {
-            'workload': f'{args.config}: {cfg["n"]} x {cfg["d"]} unit-norm '
+            'workload': f'{args.config}: {cfg["n"]} x {cfg["d"]} '
+                        f'{"unit-norm " if cfg["normalize"] else ""}'
                         f'{cfg["n_centers"]}-component mixture, dp={dp}, '
                         f'sample_ratio={cfg["ratio"]}, {cfg["graph"]}, '
                         f'{cfg["entry"]}, {B} queries, top-{k}',

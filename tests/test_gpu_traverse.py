@@ -135,3 +135,71 @@ def test_argument_errors(device):
     with pytest.raises(RuntimeError):
         kernels.traverse_cuda(**{**args, 'n_neighbors': 16})
     torch.cuda.synchronize()
+
+
+def test_edge_shapes(device):
+    """Empty batch, a single query, one result slot per beam, no entries,
+    entries that all lack a storage row, degree 1, n_storage not a multiple
+    of 32."""
+    p = Problem(n=1003, d=16, deg=8, sample_ratio=0.5, seed=13, n_query=5)
+    dev_args = dict(indptr=p.sub_indptr.to(device), indices=p.sub_indices.to(device),
+                    mapping=p.mapping.to(device),
+                    storage=p.x[p.nodelist].contiguous().to(device), n_neighbors=8)
+
+    def run(query, init_I, init_D, ef):
+        B = query.size(0)
+        out_I = torch.full((B, 4, ef), -7, dtype=torch.long, device=device)
+        out_D = torch.full((B, 4, ef), -7.0, dtype=torch.float, device=device)
+        kernels.traverse_cuda(output_I=out_I, output_D=out_D, query=query.to(device),
+                              initial_I=init_I.to(device), initial_D=init_D.to(device),
+                              **dev_args)
+        torch.cuda.synchronize()
+        ref_I = np.empty((B, 4 * ef), np.int64)
+        ref_D = np.empty((B, 4 * ef), np.float32)
+        if B:
+            oracle.traverse_cpu(ref_I, ref_D, init_I.numpy().copy(), init_D.numpy().copy(),
+                                p.sub_indptr.numpy(), p.sub_indices.numpy(), p.x.numpy(),
+                                query.numpy(), 4 * ef)
+        return out_I.flatten(1).cpu().numpy(), out_D.flatten(1).cpu().numpy(), ref_I, ref_D
+
+    init_I, init_D = p.entries(4, seed=2)
+    # empty batch: nothing is launched, nothing is written
+    run(p.query[:0], init_I[:0], init_D[:0], 4)
+    for B, ef in [(1, 1), (5, 1), (5, 3), (3, 5)]:
+        I, D, rI, rD = run(p.query[:B], init_I[:B], init_D[:B], ef)
+        assert_same_search(I, D, rI, rD)
+    # no entries at all: every slot stays empty
+    none_I = torch.empty(5, 0, dtype=torch.long)
+    none_D = torch.empty(5, 0)
+    I, D, rI, rD = run(p.query, none_I, none_D, 2)
+    assert (I == -1).all() and np.isposinf(D).all()
+    assert_same_search(I, D, rI, rD)
+    # entries without a storage row only: they are popped, expanded to
+    # nothing and merged at the end
+    outside = torch.nonzero(p.mapping < 0).flatten()[:6]
+    lone_I = outside.unsqueeze(0).expand(5, -1).contiguous()
+    lone_D = (p.query.unsqueeze(1) - p.x[lone_I]).square().sum(-1).contiguous()
+    I, D, rI, rD = run(p.query, lone_I, lone_D, 2)
+    assert_same_search(I, D, rI, rD)
+    assert sorted(I[0][:6].tolist()) == sorted(outside.tolist())
+
+
+def test_degree_one_chain(device):
+    """A chain with one neighbour per node and the query beyond its end: the
+    iteration cap min(1024, 2 * 4 * ef) decides how far the search gets
+    (traverse_cpu.cpp:18,82)."""
+    n, ef = 300, 8
+    indptr = torch.arange(n + 1)
+    indices = torch.cat([torch.arange(1, n), torch.tensor([-1])])
+    x = torch.zeros(n, 8)
+    x[:, 0] = torch.arange(n).float()
+    q = torch.zeros(1, 8)
+    q[0, 0] = n + 10.0
+    out_I = torch.empty(1, 4, ef, dtype=torch.long, device=device)
+    out_D = torch.empty(1, 4, ef, dtype=torch.float, device=device)
+    kernels.traverse_cuda(out_I, out_D, indptr.to(device), indices.to(device),
+                          torch.arange(n).to(device), x.to(device), q.to(device),
+                          torch.zeros(1, 1, dtype=torch.long, device=device),
+                          torch.full((1, 1), float((n + 10) ** 2), device=device), 1)
+    cap = 2 * 4 * ef
+    assert out_I.flatten().tolist() == [cap - i for i in range(4 * ef)]
