@@ -151,20 +151,30 @@ struct OpenList {
         }
         return uni(lv[j - kRegNodes]);
     }
+    // lane l of a key bank and of its value bank := two uniform values
+    // (v_writelane takes one scalar register besides M0, which holds the lane)
+    __device__ __forceinline__ static void set_lane(int &kbank, int &vbank, int k,
+                                                    int v, int l) {
+        asm("s_mov_b32 m0, %4\n\t"
+            "s_nop 0\n\t"
+            "v_writelane_b32 %0, %2, m0\n\t"
+            "v_writelane_b32 %1, %3, m0"
+            : "+v"(kbank), "+v"(vbank)
+            : "s"(k), "s"(v), "s"(l)
+            : "m0");
+    }
     __device__ __forceinline__ void put(const int KIND, int j, int k, int v,
                                         int lane) {
         if (KIND == 0) {
-            const bool mine = lane == j;
-            Ak = mine ? k : Ak, Av = mine ? v : Av;
+            set_lane(Ak, Av, k, v, j);
         } else if (KIND == 1) {
-            const bool mine = lane == j - 64;
-            Bk = mine ? k : Bk, Bv = mine ? v : Bv;
+            set_lane(Bk, Bv, k, v, j - 64);
         } else if (KIND == 2) {
-            const bool mine = lane == ((j - 128) >> 1);
+            const int l = (j - 128) >> 1;
             if (j & 1) {
-                Dk = mine ? k : Dk, Dv = mine ? v : Dv;
+                set_lane(Dk, Dv, k, v, l);
             } else {
-                Ck = mine ? k : Ck, Cv = mine ? v : Cv;
+                set_lane(Ck, Cv, k, v, l);
             }
         } else if (lane == 0) {
             lk[j - kRegNodes] = k, lv[j - kRegNodes] = v;
