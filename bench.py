@@ -311,6 +311,29 @@ def main():
                                  counts)),
         },
     }
+    # context, not part of `value`: the same step with its inputs and outputs
+    # crossing PCIe (pageable host memory), and the whole three-stage search
+    # (`IndexStaged.search`: rotation on the host, entries, pipeline).
+    host_q = stage.query_rot[:, :dp].contiguous()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(3):
+        stage.query_cuda.copy_(host_q)
+        oI, oD = stage.step(ef)
+        oI.cpu(), oD.cpu()
+    line['config']['ms_per_step_with_pcie'] = round(
+        1e3 * (time.perf_counter() - t0) / 3, 3)
+    chunk = 1000 if B % 1000 == 0 else B
+    index.search(query, k=k, ef_search=ef, chunk_size=chunk)
+    t0 = time.perf_counter()
+    top_I, _ = index.search(query, k=k, ef_search=ef, chunk_size=chunk)
+    t_e2e = time.perf_counter() - t0
+    from pilotann_amd import utils as _utils
+    line['config']['end_to_end'] = {
+        'api': 'IndexStaged.search', 'chunk_size': chunk,
+        'queries_per_s': round(B / t_e2e, 1),
+        'recall_at_10': round(_utils.recall(top_I, target), 4)}
+
     if not args.no_cpu_baseline:
         EP_I, EP_D = stage.entries()
         torch.cuda.synchronize()

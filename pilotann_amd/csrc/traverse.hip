@@ -12,18 +12,22 @@
 //     what the reference's result heap holds — spread over registers,
 //     ceil(H/64) entries per lane;
 //   * the visited set is exact: one bit per storage row in a per-wavefront
-//     slice of a pooled HBM bitmask, tested and set with one atomic OR per
-//     neighbour;
+//     slice of a pooled HBM bitmask (atomic OR), behind a small LDS table of
+//     rows already known to be marked;
 //   * a distance is the reference's eight-accumulator FMA sum
 //     (extension/inc/distance.h:31-55) bit for bit: four lanes share a row,
 //     lane a of the quad owns accumulators 2a and 2a+1 and streams its 8
 //     bytes of every 32-byte group.
-// Expansion of a node therefore costs one coalesced row of neighbour ids, one
-// atomic per neighbour and one coalesced 4*dp-byte row per unvisited
-// neighbour, 16 rows in flight per pass.
+// Expansion of a node therefore costs one coalesced row of neighbour ids, an
+// atomic for each neighbour the LDS table does not know and one coalesced
+// 4*dp-byte row per unvisited neighbour, 16 rows in flight per pass.
 #include <hip/hip_runtime.h>
 #include <math.h>
 #include <stdint.h>
+
+#include <map>
+#include <mutex>
+#include <tuple>
 
 #include "device_common.h"
 #include "pilotann.h"
@@ -803,12 +807,26 @@ int make_plan(int64_t n_storage, int64_t batch, int dp, int ef_total, Plan *p) {
     if (!p->fn) return PA_E_EF;
     int dev = 0, cus = 0, per_cu = 0;
     hipError_t e = hipGetDevice(&dev);
-    if (e == hipSuccess)
-        e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
-    if (e == hipSuccess)
-        e = hipOccupancyMaxActiveBlocksPerMultiprocessor(
-            &per_cu, reinterpret_cast<const void *>(p->fn), kWave, p->lds_bytes);
     if (e != hipSuccess) return (int)e;
+    {
+        // the residency of a (device, kernel, LDS size) never changes
+        static std::mutex mutex;
+        static std::map<std::tuple<int, const void *, int>, std::pair<int, int>> known;
+        std::lock_guard<std::mutex> guard(mutex);
+        const auto key = std::make_tuple(
+            dev, reinterpret_cast<const void *>(p->fn), p->lds_bytes);
+        auto it = known.find(key);
+        if (it == known.end()) {
+            e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+            if (e == hipSuccess)
+                e = hipOccupancyMaxActiveBlocksPerMultiprocessor(
+                    &per_cu, reinterpret_cast<const void *>(p->fn), kWave,
+                    p->lds_bytes);
+            if (e != hipSuccess) return (int)e;
+            it = known.emplace(key, std::make_pair(cus, per_cu)).first;
+        }
+        cus = it->second.first, per_cu = it->second.second;
+    }
     if (per_cu < 1) per_cu = 1;
     int64_t slots = (int64_t)per_cu * cus;
     if (slots < 1) slots = 1;
@@ -901,7 +919,7 @@ extern "C" int pa_traverse(int64_t *out_I, float *out_D, const int32_t *adj,
                            void *stream_) {
     if (batch < 0 || n_nodes <= 0 || n_init < 0 || beam < 1 || ef < 1)
         return PA_E_SHAPE;
-    if (n_nodes >= (1ll << 31)) return PA_E_RANGE;
+    if (n_nodes >= (1ll << 31) || batch >= (1ll << 31)) return PA_E_RANGE;
     if (n_neighbors < 1 || n_neighbors > PA_MAX_NEIGHBORS) return PA_E_NEIGHBORS;
     if ((int64_t)beam * ef > PA_MAX_EF_TOTAL) return PA_E_EF;
     Plan p;
