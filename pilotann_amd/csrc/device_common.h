@@ -92,20 +92,29 @@ __device__ __forceinline__ float quad_square_dist(const float2 *row,
     float a0 = 0.f, a1 = 0.f;
     if (active) {
         if (DP8) {
-            // all loads of the row first; the query is then read from LDS
-            // four groups at a time (the fences keep the compiler from
-            // hoisting those reads, which would double the live registers)
-            float2 x[DP8 ? DP8 : 1];
+            // All loads of a batch first, then the query from LDS four groups
+            // at a time (the fences keep the compiler from hoisting those
+            // reads, which would double the live registers).  PA_ROW_SPLIT
+            // batches per row: 1 keeps a whole row in flight.
+#ifndef PA_ROW_SPLIT
+#define PA_ROW_SPLIT 1
+#endif
+            constexpr int kBatch = DP8 >= 4 * PA_ROW_SPLIT ? DP8 / PA_ROW_SPLIT : (DP8 ? DP8 : 1);
 #pragma unroll
-            for (int t = 0; t < DP8; ++t) x[t] = row[4 * t];
-            __builtin_amdgcn_sched_barrier(0);
+            for (int h = 0; h < (DP8 ? DP8 : 1); h += kBatch) {
+                float2 x[kBatch];
 #pragma unroll
-            for (int t = 0; t < DP8; ++t) {
-                const float2 y = qv[4 * t];
-                const float d0 = y.x - x[t].x, d1 = y.y - x[t].y;
-                a0 = fmaf(d0, d0, a0);
-                a1 = fmaf(d1, d1, a1);
-                if ((t & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+                for (int t = 0; t < kBatch; ++t) x[t] = row[4 * (h + t)];
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int t = 0; t < kBatch; ++t) {
+                    const float2 y = qv[4 * (h + t)];
+                    const float d0 = y.x - x[t].x, d1 = y.y - x[t].y;
+                    a0 = fmaf(d0, d0, a0);
+                    a1 = fmaf(d1, d1, a1);
+                    if ((t & 3) == 3) __builtin_amdgcn_sched_barrier(0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
         } else {
 #pragma unroll 4

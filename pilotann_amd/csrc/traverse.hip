@@ -38,7 +38,10 @@ namespace {
 
 constexpr int kSlotAlignWords = 256;   // bitmask slice: multiple of 1 KiB
 constexpr int kWorkCounterBytes = 256; // head of the workspace
-constexpr int kSeenCacheLog2 = 10;
+#ifndef PA_SEEN_LOG2
+#define PA_SEEN_LOG2 10
+#endif
+constexpr int kSeenCacheLog2 = PA_SEEN_LOG2;
 constexpr int kSeenCache = 1 << kSeenCacheLog2;  // LDS words remembering visited rows
 
 // ---- open list: heapq.cuh, top of the heap in registers ----------------------
@@ -180,7 +183,10 @@ struct OpenList {
             } else {
                 set_lane(Ck, Cv, k, v, l);
             }
-        } else if (lane == 0) {
+        } else {
+            // every lane stores the same pair to the same cell: one LDS
+            // write, and no divergent branch around it
+            (void)lane;
             lk[j - kRegNodes] = k, lv[j - kRegNodes] = v;
         }
     }
