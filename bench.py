@@ -11,7 +11,7 @@ line is printed; `value` is queries per second of that step.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W]
                     [--n-base N] [--queries B] [--ef EF] [--no-cpu-baseline]
-                    [--copy-calibration]
+                    [--no-context] [--copy-calibration]
 """
 import argparse
 import contextlib
@@ -204,6 +204,11 @@ def main():
     ap.add_argument('--queries', type=int, default=None)
     ap.add_argument('--ef', type=int, default=None)
     ap.add_argument('--no-cpu-baseline', action='store_true')
+    ap.add_argument('--no-context', action='store_true',
+                    help='skip the context figures (PCIe-inclusive step, '
+                         'fourfold batch, end-to-end search), so that a '
+                         'kernel trace of the run holds the timed launches '
+                         'only')
     ap.add_argument('--copy-calibration', action='store_true',
                     help='only run a plain 1 GiB device copy five times (to '
                          'scale the FETCH_SIZE / WRITE_SIZE counters) and exit')
@@ -311,9 +316,27 @@ def main():
                                  counts)),
         },
     }
-    # context, not part of `value`: the same step with its inputs and outputs
-    # crossing PCIe (pageable host memory), and the whole three-stage search
-    # (`IndexStaged.search`: rotation on the host, entries, pipeline).
+    if not args.no_context:
+        context_figures(line, args, cfg, index, stage, query, target, ef,
+                        launch_bytes, out_D)
+
+    if not args.no_cpu_baseline:
+        EP_I, EP_D = stage.entries()
+        torch.cuda.synchronize()
+        base, (ref_I, ref_D, n) = cpu_baseline(index, stage, ef, EP_I, EP_D)
+        line['cpu_baseline'] = base
+        same = (np.array_equal(out_D.flatten(1)[:n].cpu().numpy(), ref_D))
+        line['config']['matches_cpu_baseline'] = bool(same)
+    print(json.dumps(line), flush=True)
+
+
+def context_figures(line, args, cfg, index, stage, query, target, ef,
+                    launch_bytes, out_D):
+    """Not part of `value`: the same step with its inputs and outputs
+    crossing PCIe (pageable host memory), the launch over a fourfold batch,
+    and the whole three-stage search (`IndexStaged.search`: rotation on the
+    host, entries, pipeline)."""
+    B, k, dp, device = stage.B, cfg['k'], cfg['dp'], stage.device
     host_q = stage.query_rot[:, :dp].contiguous()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -323,6 +346,34 @@ def main():
         oI.cpu(), oD.cpu()
     line['config']['ms_per_step_with_pcie'] = round(
         1e3 * (time.perf_counter() - t0) / 3, 3)
+    # context: the same launch over four copies of the batch.  One launch
+    # keeps 5120 independent searches in flight; filling and draining them
+    # weighs less on a longer batch, which shows the kernel's marginal rate.
+    rep = 4
+    big_q = stage.query_cuda.repeat(rep, 1).contiguous()
+    big_EI, big_ED = [t.repeat(rep, 1).contiguous() for t in stage.entries()]
+    big_I = torch.empty(rep * B, 4, ef, dtype=torch.long, device=device)
+    big_D = torch.empty(rep * B, 4, ef, dtype=torch.float, device=device)
+    big_ev = []
+    for i in range(4):
+        a, b = (torch.cuda.Event(enable_timing=True) for _ in range(2))
+        a.record()
+        stage.kernels.traverse_prepared(big_I, big_D, stage.graph,
+                                        index.storage_cuda, big_q, big_EI,
+                                        big_ED, None)
+        b.record()
+        big_ev.append((a, b))
+    torch.cuda.synchronize()
+    big_ms = float(np.mean([a.elapsed_time(b) for a, b in big_ev[1:]]))
+    big_rate = rep * launch_bytes / (big_ms * 1e-3) / 1e9
+    line['config']['batch_x4'] = {
+        'queries': rep * B, 'kernel_ms': round(big_ms, 4),
+        'queries_per_s': round(rep * B / (big_ms * 1e-3), 1),
+        'achieved_GBps': round(big_rate, 1),
+        'frac': round(big_rate / HBM_PEAK_GBS, 4),
+        'same_results': bool(torch.equal(big_D[-B:], out_D))}
+    del big_q, big_EI, big_ED, big_I, big_D
+
     chunk = 1000 if B % 1000 == 0 else B
     index.search(query, k=k, ef_search=ef, chunk_size=chunk)
     t0 = time.perf_counter()
@@ -333,15 +384,6 @@ def main():
         'api': 'IndexStaged.search', 'chunk_size': chunk,
         'queries_per_s': round(B / t_e2e, 1),
         'recall_at_10': round(_utils.recall(top_I, target), 4)}
-
-    if not args.no_cpu_baseline:
-        EP_I, EP_D = stage.entries()
-        torch.cuda.synchronize()
-        base, (ref_I, ref_D, n) = cpu_baseline(index, stage, ef, EP_I, EP_D)
-        line['cpu_baseline'] = base
-        same = (np.array_equal(out_D.flatten(1)[:n].cpu().numpy(), ref_D))
-        line['config']['matches_cpu_baseline'] = bool(same)
-    print(json.dumps(line), flush=True)
 
 
 if __name__ == '__main__':

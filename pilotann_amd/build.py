@@ -19,7 +19,7 @@ HIP_FLAGS = [
     # packed fp32 instructions off (device pass; the host pass warns that it
     # does not know the feature, which is harmless)
     '-Xclang', '-target-feature', '-Xclang', '-packed-fp32-ops',
-    '-Wno-unused-command-line-argument',
+    '-Wno-unused-command-line-argument', '-Wno-inline-asm',
 ]
 # the reference's host flags (setup.py:39-44) minus -ffast-math: the host
 # search must add in the order it is written

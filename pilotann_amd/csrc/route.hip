@@ -56,7 +56,6 @@ __global__ __launch_bounds__(kWave) void route_score_kernel(
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[r] = 0.f;
         float norm = 0.f;
-#pragma unroll 4
         for (int c = 0; c < groups; ++c) {
             float4 a = qrow[2 * c];
             float4 b = rrow[2 * c];

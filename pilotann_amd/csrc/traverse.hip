@@ -541,7 +541,7 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
                 const int cell = v & (kSeenCache - 1);
                 const uint32_t tag = (uint32_t)v >> kSeenCacheLog2;
                 const uint32_t ways = use_cache ? seen_cache[cell] : 0xffffffffu;
-                if ((ways & 0xffffu) != tag && (ways >> 16) != tag) {
+                if (!use_cache || ((ways & 0xffffu) != tag && (ways >> 16) != tag)) {
                     before = atomicOr(&seen[v >> 5], 1u << (v & 31));
                     if (use_cache) seen_cache[cell] = (ways << 16) | tag;
                 }
