@@ -144,8 +144,11 @@ struct OpenList {
         if (KIND == 0) return rl(Ak, j);
         if (KIND == 1) return rl(Bk, j - 64);
         if (KIND == 2) {
+            // both banks are read and one result is kept: two instructions
+            // more than a branch on the parity of j would need, no branch
             const int l = (j - 128) >> 1;
-            return (j & 1) ? rl(Dk, l) : rl(Ck, l);
+            const int left = rl(Ck, l), right = rl(Dk, l);
+            return (j & 1) ? right : left;
         }
         return uni(lk[j - kRegNodes]);
     }
@@ -154,7 +157,8 @@ struct OpenList {
         if (KIND == 1) return rl(Bv, j - 64);
         if (KIND == 2) {
             const int l = (j - 128) >> 1;
-            return (j & 1) ? rl(Dv, l) : rl(Cv, l);
+            const int left = rl(Cv, l), right = rl(Dv, l);
+            return (j & 1) ? right : left;
         }
         return uni(lv[j - kRegNodes]);
     }
@@ -177,16 +181,18 @@ struct OpenList {
         } else if (KIND == 1) {
             set_lane(Bk, Bv, k, v, j - 64);
         } else if (KIND == 2) {
+            // lane-masked selects on both banks instead of a branch on the
+            // parity of j around two v_writelane
             const int l = (j - 128) >> 1;
-            if (j & 1) {
-                set_lane(Dk, Dv, k, v, l);
-            } else {
-                set_lane(Ck, Cv, k, v, l);
-            }
+            const bool here = lane == l;
+            const bool right = j & 1;
+            Ck = (here && !right) ? k : Ck;
+            Cv = (here && !right) ? v : Cv;
+            Dk = (here && right) ? k : Dk;
+            Dv = (here && right) ? v : Dv;
         } else {
             // every lane stores the same pair to the same cell: one LDS
             // write, and no divergent branch around it
-            (void)lane;
             lk[j - kRegNodes] = k, lv[j - kRegNodes] = v;
         }
     }
@@ -271,6 +277,7 @@ struct OpenList {
         const Choice ch = choices<true>();
         int j = 1;
         bool bottom = true;  // the walk reached level kDepth
+        int walked_key = 0;  // key of node j when its level is an LDS level
 #pragma unroll
         for (int L = 1; L <= kDepth; ++L) {
             if (L == kDepth && 2 * j > kSize) {
@@ -284,33 +291,38 @@ struct OpenList {
                 int ka, kb, va, vb;
                 pair(3, false, 2 * j, ka, kb, va, vb);
                 if (L == kDepth) kb = 2 * j == kSize ? ka : kb;
-                j = add_if_ne(2 * j, max(ka, kb), ka);
+                walked_key = max(ka, kb);
+                j = add_if_ne(2 * j, walked_key, ka);
             }
         }
-        if (k >= (bottom ? key_of(kind(kDepth), j) : key_of(kind(kDepth - 1), j)))
-            return;
-        if (bottom) {
+        // the leaf's key: the walk has it already when the leaf is in LDS
+        int leaf_key;
+        if (bottom)
+            leaf_key = kind(kDepth) == 3 ? walked_key : key_of(kind(kDepth), j);
+        else
+            leaf_key = kind(kDepth - 1) == 3 ? walked_key : key_of(kind(kDepth - 1), j);
+        if (k >= leaf_key) return;
+        // one store per level: the parent's entry while it is larger than
+        // the new key, the new entry where the rise stops
+        auto rise = [&](const int L) -> bool {
             const int up = j >> 1;
-            const int pk = key_of(kind(kDepth - 1), up);
-            if (pk <= k) {
-                put(kind(kDepth), j, k, v, lane);
-                wave_sync();
-                return;
-            }
-            put(kind(kDepth), j, pk, val_of(kind(kDepth - 1), up), lane);
+            const int pk = key_of(kind(L - 1), up);
+            const int pv = val_of(kind(L - 1), up);
+            const bool stop = pk <= k;
+            put(kind(L), j, stop ? k : pk, stop ? v : pv, lane);
             j = up;
+            return stop;
+        };
+        if (bottom && rise(kDepth)) {
+            wave_sync();
+            return;
         }
 #pragma unroll
         for (int L = kDepth - 1; L >= 1; --L) {
-            const int up = j >> 1;
-            const int pk = key_of(kind(L - 1), up);
-            if (pk <= k) {
-                put(kind(L), j, k, v, lane);
+            if (rise(L)) {
                 wave_sync();
                 return;
             }
-            put(kind(L), j, pk, val_of(kind(L - 1), up), lane);
-            j = up;
         }
         put(0, 1, k, v, lane);
         wave_sync();
