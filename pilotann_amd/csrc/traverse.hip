@@ -53,8 +53,8 @@ constexpr int kSeenCache = 1 << kSeenCacheLog2;  // LDS words remembering visite
 // Levels 0..7 live in registers, one node per lane: bank A levels 0..5 (node j
 // in lane j), bank B level 6 (lane j - 64), banks C and D the left and right
 // children of level 7 (lane (j - 128) / 2), so a sibling pair is always two
-// v_readlane of known registers.  Deeper nodes sit in LDS at [j - 256], a
-// sibling pair per aligned 8 bytes.  Keys are kept as order-preserving
+// v_readlane of known registers.  Deeper nodes sit in LDS at [j - 256] as
+// (key, value), a sibling pair per aligned 16 bytes.  Keys are kept as order-preserving
 // integers (float_to_key) so that every comparison of a walk is a scalar
 // integer compare.  All lanes run the same, uniform, control flow; the walks
 // are unrolled by level so that each level is a dozen instructions.  After
@@ -98,8 +98,7 @@ struct OpenList {
     static constexpr int kLdsCells = kSize + 2 > kRegNodes ? kSize + 2 - kRegNodes : 0;
     static constexpr int kInf = 0x7f800000;       // float_to_key(+inf)
     int Ak, Av, Bk, Bv, Ck, Cv, Dk, Dv;
-    int *lk;  // node j >= 256 at [j - 256]
-    int *lv;
+    int2 *cells;  // node j >= 256 at [j - 256] as (key, value); 16-byte aligned
 
     __device__ __forceinline__ static int rl(int x, int l) {
         return __builtin_amdgcn_readlane(x, l);
@@ -112,7 +111,7 @@ struct OpenList {
     __device__ __forceinline__ void reset(int lane) {
         Ak = Bk = Ck = Dk = kInf;
         Av = Bv = Cv = Dv = -1;
-        for (int i = lane; i < kLdsCells; i += kWave) lk[i] = kInf, lv[i] = -1;
+        for (int i = lane; i < kLdsCells; i += kWave) cells[i] = make_int2(kInf, -1);
     }
 
     // keys (and values) of the sibling pair (c, c + 1), c even, of a level.
@@ -132,12 +131,10 @@ struct OpenList {
             ka = rl(Ck, l), kb = rl(Dk, l);
             if (VALS) va = rl(Cv, l), vb = rl(Dv, l);
         } else {
-            const int2 k2 = *reinterpret_cast<const int2 *>(lk + (c - kRegNodes));
-            if (VALS) {
-                const int2 v2 = *reinterpret_cast<const int2 *>(lv + (c - kRegNodes));
-                va = uni(v2.x), vb = uni(v2.y);
-            }
-            ka = uni(k2.x), kb = uni(k2.y);
+            // one 16-byte read: both children with their values
+            const int4 p = *reinterpret_cast<const int4 *>(cells + (c - kRegNodes));
+            if (VALS) va = uni(p.y), vb = uni(p.w);
+            ka = uni(p.x), kb = uni(p.z);
         }
     }
     __device__ __forceinline__ int key_of(const int KIND, int j) const {
@@ -150,7 +147,7 @@ struct OpenList {
             const int left = rl(Ck, l), right = rl(Dk, l);
             return (j & 1) ? right : left;
         }
-        return uni(lk[j - kRegNodes]);
+        return uni(cells[j - kRegNodes].x);
     }
     __device__ __forceinline__ int val_of(const int KIND, int j) const {
         if (KIND == 0) return rl(Av, j);
@@ -160,7 +157,7 @@ struct OpenList {
             const int left = rl(Cv, l), right = rl(Dv, l);
             return (j & 1) ? right : left;
         }
-        return uni(lv[j - kRegNodes]);
+        return uni(cells[j - kRegNodes].y);
     }
     // lane l of a key bank and of its value bank := two uniform values
     // (v_writelane takes one scalar register besides M0, which holds the lane)
@@ -193,7 +190,7 @@ struct OpenList {
         } else {
             // every lane stores the same pair to the same cell: one LDS
             // write, and no divergent branch around it
-            lk[j - kRegNodes] = k, lv[j - kRegNodes] = v;
+            cells[j - kRegNodes] = make_int2(k, v);
         }
     }
 
@@ -456,7 +453,7 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
     float *okey = reinterpret_cast<float *>(smem);
     int *oval = reinterpret_cast<int *>(okey + heap_cells);
     OpenList<H> open;
-    open.lk = reinterpret_cast<int *>(okey), open.lv = oval;
+    open.cells = reinterpret_cast<int2 *>(smem);
     int *cand_id = oval + heap_cells;
     float *cand_key = reinterpret_cast<float *>(cand_id + kWave);
     float *qv = cand_key + kWave;
