@@ -1,0 +1,126 @@
+"""Seeded sweep of the traversal over random graphs and shapes: every heap
+size of the ladder, vector lengths with and without a specialised kernel,
+degrees 1..64, ragged rows, self loops, repeated neighbours, neighbours and
+entries without a storage row.  Bar as everywhere: distances bit-identical to
+the oracle, ids identical except inside exact ties."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from pilotann_amd import kernels
+from common import assert_same_search
+
+pytestmark = pytest.mark.gpu
+
+EF = [4, 8, 12, 16, 24, 32, 48, 64, 96, 128, 256, 512]      # 4*ef = the ladder
+DP = [8, 16, 24, 32, 40, 64, 72, 128, 200, 256]
+
+
+def make_case(seed):
+    r = np.random.RandomState(seed)
+    n_nodes = int(r.randint(300, 5000))
+    ratio = float(r.choice([0.3, 0.6, 1.0]))
+    n_rows = max(8, int(n_nodes * ratio))
+    deg = int(r.choice([1, 2, 3, 7, 16, 24, 31, 32, 33, 48, 63, 64]))
+    dp = int(r.choice(DP))
+    ef = int(r.choice(EF))
+    n_init = int(r.choice([1, 3, 16, 32, 64, 100]))
+    B = int(r.randint(1, 70))
+    g = torch.Generator().manual_seed(seed)
+    nodelist = torch.randperm(n_nodes, generator=g)[:n_rows].sort().values
+    mapping = torch.full((n_nodes,), -1, dtype=torch.long)
+    mapping[nodelist] = torch.arange(n_rows)
+    # neighbours drawn from all nodes with a bias to a window, so that rows
+    # repeat ids, hit the node itself and (for ratio < 1) unsampled nodes
+    base = nodelist.unsqueeze(1) + torch.randint(-20, 21, (n_rows, deg), generator=g)
+    far = torch.randint(n_nodes, (n_rows, deg), generator=g)
+    pick = torch.rand(n_rows, deg, generator=g) < 0.5
+    nbr = torch.where(pick, base.clamp(0, n_nodes - 1), far)
+    if ratio == 1.0 or r.rand() < 0.5:
+        # the host search reads a vector for every neighbour: keep them sampled
+        nbr = nodelist[torch.searchsorted(nodelist, nbr).clamp(max=n_rows - 1)]
+        unsampled_neighbours = False
+    else:
+        unsampled_neighbours = True
+    length = torch.randint(0, deg + 1, (n_rows, 1), generator=g)
+    nbr[torch.arange(deg).unsqueeze(0) >= length] = -1
+    rowlen = torch.zeros(n_nodes, dtype=torch.long)
+    rowlen[nodelist] = deg
+    indptr = torch.zeros(n_nodes + 1, dtype=torch.long)
+    indptr[1:] = torch.cumsum(rowlen, 0)
+    x = torch.randn(n_nodes, dp, generator=g)
+    tied = r.rand() < 0.3
+    if tied:
+        x = (x * 2).round() / 2          # many exact ties
+    query = torch.randn(B, dp, generator=g)
+    init_I = torch.randint(n_nodes, (B, n_init), generator=g)
+    if r.rand() < 0.5:
+        init_I = nodelist[torch.randint(n_rows, (B, n_init), generator=g)]
+    return dict(seed=seed, n_nodes=n_nodes, n_rows=n_rows, deg=deg, dp=dp, ef=ef,
+                n_init=n_init, B=B, nodelist=nodelist, mapping=mapping,
+                indptr=indptr, indices=nbr.flatten().contiguous(), x=x,
+                query=query, init_I=init_I.contiguous(), tied=tied,
+                unsampled_neighbours=unsampled_neighbours)
+
+
+@pytest.mark.parametrize('seed', range(150))
+def test_random_graph(seed, device):
+    c = make_case(1000 + seed)
+    print('fuzz', {k: c[k] for k in ('seed', 'n_nodes', 'n_rows', 'deg', 'dp',
+                                     'ef', 'n_init', 'B', 'tied',
+                                     'unsampled_neighbours')},
+          flush=True)
+    B, k = c['B'], 4 * c['ef']
+    xn, qn = c['x'].numpy(), c['query'].numpy()
+    init_D = torch.from_numpy(np.stack([
+        oracle.square_dist(qn[b].copy(), xn, c['init_I'][b].numpy().copy())
+        for b in range(B)]))
+    indices = c['indices']
+    if c['unsampled_neighbours']:
+        # the device skips neighbours without a storage row; give the oracle
+        # the same graph with those entries taken out of their rows
+        rows = indices.view(c['n_rows'], c['deg']).clone()
+        ok = (rows >= 0) & (c['mapping'][rows.clamp(min=0)] >= 0)
+        first_neg = torch.where((rows < 0).any(1), (rows < 0).float().argmax(1),
+                                torch.full((rows.size(0),), c['deg']))
+        ok &= torch.arange(c['deg']).unsqueeze(0) < first_neg.unsqueeze(1)
+        order = torch.argsort((~ok).to(torch.int8), dim=1, stable=True)
+        rows = torch.where(torch.gather(ok, 1, order), torch.gather(rows, 1, order),
+                           torch.full_like(rows, -1))
+        oracle_indices = rows.flatten().contiguous()
+    else:
+        oracle_indices = indices
+    ref_I = np.empty((B, k), np.int64)
+    ref_D = np.empty((B, k), np.float32)
+    oracle.traverse_cpu(ref_I, ref_D, c['init_I'].numpy().copy(),
+                        init_D.numpy().copy(), c['indptr'].numpy(),
+                        oracle_indices.numpy(), xn, qn, k)
+    out_I = torch.empty(B, 4, c['ef'], dtype=torch.long, device=device)
+    out_D = torch.empty(B, 4, c['ef'], dtype=torch.float, device=device)
+    kernels.traverse_cuda(
+        output_I=out_I, output_D=out_D, indptr=c['indptr'].to(device),
+        indices=indices.to(device), mapping=c['mapping'].to(device),
+        storage=c['x'][c['nodelist']].contiguous().to(device),
+        query=c['query'].to(device), initial_I=c['init_I'].to(device),
+        initial_D=init_D.to(device), n_neighbors=c['deg'])
+    torch.cuda.synchronize()
+    got_I = out_I.flatten(1).cpu().numpy()
+    got_D = out_D.flatten(1).cpu().numpy()
+    if not c['tied']:
+        assert_same_search(got_I, got_D, ref_I, ref_D)
+        return
+    # With exact ties among the kept distances the two result lists may keep
+    # different members of a tie (which of several equally bad entries leaves
+    # first has no effect on the search).  Distances still agree bit for bit;
+    # an id that differs must be a row at exactly the reported distance, and
+    # ids repeat only as often as in the oracle's list (repeated entries).
+    assert np.array_equal(got_D, ref_D)
+    for b in range(B):
+        ids, ref_ids = got_I[b][got_I[b] >= 0], ref_I[b][ref_I[b] >= 0]
+        assert len(ids) - len(set(ids.tolist())) == len(ref_ids) - len(set(ref_ids.tolist()))
+        diff = np.flatnonzero(got_I[b] != ref_I[b])
+        if len(diff):
+            assert (got_I[b][diff] >= 0).all()
+            true_d = oracle.square_dist(qn[b].copy(), xn, got_I[b][diff].copy())
+            assert np.array_equal(true_d, got_D[b][diff])
