@@ -68,3 +68,31 @@ def test_routing_argument_errors(device):
                              ev[:, :24].contiguous())
     with pytest.raises(RuntimeError):
         kernels.routing_cuda(q, rv, en.int(), ev)
+
+
+@pytest.mark.parametrize('seed', range(24))
+def test_routing_random_shapes(seed, device):
+    r = np.random.RandomState(500 + seed)
+    R = int(r.choice([1, 2, 5, 31, 32, 33, 64, 100, 257]))
+    L = int(r.choice([32, 64, 128]))
+    d = int(r.choice([8, 24, 40, 64, 128, 256]))
+    B = int(r.randint(1, 1500))
+    print('route', dict(R=R, L=L, d=d, B=B), flush=True)
+    g = torch.Generator().manual_seed(seed)
+    q = torch.rand(B, d, generator=g)
+    route_vectors = torch.rand(R, d, generator=g)
+    entry_vectors = torch.rand(R, L, d, generator=g)
+    entry_nodes = torch.arange(R * L).view(R, L)
+    router, dist = kernels.routing_cuda(
+        q.to(device), route_vectors.to(device), entry_nodes.to(device),
+        entry_vectors.to(device))
+    router, dist = router.cpu().numpy(), dist.cpu().numpy()
+    assert router.min() >= 0 and router.max() < R
+    exact = torch.cdist(q.double(), route_vectors.double()).square().numpy()
+    chosen = exact[np.arange(B), router]
+    assert (chosen <= exact.min(-1) * (1 + 1e-5) + 1e-6).all()
+    flat = entry_vectors.view(R * L, d).numpy()
+    ref = np.stack([
+        oracle.square_dist(q[b].numpy(), flat, entry_nodes[router[b]].numpy().copy())
+        for b in range(B)])
+    assert np.array_equal(dist, ref)
