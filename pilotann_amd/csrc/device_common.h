@@ -78,12 +78,22 @@ __device__ __forceinline__ int wave_max_key(int x) {
 // accumulators are then added left to right.  Four adjacent lanes (a quad)
 // share a row: lane a of the quad owns accumulators 2a and 2a + 1 and streams
 // its 8 bytes of every 32-byte group, so all loads of a row are in flight at
-// once in 2 * dp / 8 registers.  `row` and `qv` already point at the lane's
-// pair of the first group.  Lane 0 of the quad returns the distance; every
+// once in 2 * dp / 8 registers.  `row` points at the lane's pair of the first
+// group, `qv` at the lane's run of the query in LDS (query_slot layout).  Lane 0 of the quad returns the distance; every
 // lane of the wavefront must call this (the exchange inside the quad is a DPP
 // move), lanes without a row pass active = false.
 constexpr int kLanesPerRow = 4;
 constexpr int kRowsPerPass = kWave / kLanesPerRow;
+
+// Where element i of a query goes in LDS: the 8-byte pairs one lane of a quad
+// needs (pair a of every group of eight) lie next to each other, so that two
+// groups are one 16-byte read; two pairs of padding after each lane's run keep
+// the four runs on different banks.  `groups` = dp / 8.
+__host__ __device__ constexpr int query_run(int groups) { return groups + 2; }
+__host__ __device__ constexpr int query_floats(int dp) { return 8 * query_run(dp >> 3); }
+__device__ __forceinline__ int query_slot(int i, int groups) {
+    return 2 * (((i >> 1) & 3) * query_run(groups) + (i >> 3)) + (i & 1);
+}
 
 template <int DP8>
 __device__ __forceinline__ float quad_square_dist(const float2 *row,
@@ -91,36 +101,34 @@ __device__ __forceinline__ float quad_square_dist(const float2 *row,
                                                   bool active) {
     float a0 = 0.f, a1 = 0.f;
     if (active) {
-        if (DP8) {
-            // All loads of a batch first, then the query from LDS four groups
-            // at a time (the fences keep the compiler from hoisting those
-            // reads, which would double the live registers).  PA_ROW_SPLIT
-            // batches per row: 1 keeps a whole row in flight.
-#ifndef PA_ROW_SPLIT
-#define PA_ROW_SPLIT 1
-#endif
-            constexpr int kBatch = DP8 >= 4 * PA_ROW_SPLIT ? DP8 / PA_ROW_SPLIT : (DP8 ? DP8 : 1);
+        if (DP8 > 0 && DP8 % 2 == 0) {
+            // All loads of the row first, then the query from LDS, 16 bytes
+            // (two groups) per read, four groups at a time (the fences keep
+            // the compiler from hoisting those reads, which would double the
+            // live registers).
+            constexpr int kPairs = DP8 > 0 ? DP8 : 2;
+            float2 x[kPairs];
 #pragma unroll
-            for (int h = 0; h < (DP8 ? DP8 : 1); h += kBatch) {
-                float2 x[kBatch];
+            for (int t = 0; t < kPairs; ++t) x[t] = row[4 * t];
+            __builtin_amdgcn_sched_barrier(0);
+            const float4 *q4 = reinterpret_cast<const float4 *>(qv);
 #pragma unroll
-                for (int t = 0; t < kBatch; ++t) x[t] = row[4 * (h + t)];
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int t = 0; t < kBatch; ++t) {
-                    const float2 y = qv[4 * (h + t)];
-                    const float d0 = y.x - x[t].x, d1 = y.y - x[t].y;
-                    a0 = fmaf(d0, d0, a0);
-                    a1 = fmaf(d1, d1, a1);
-                    if ((t & 3) == 3) __builtin_amdgcn_sched_barrier(0);
-                }
-                __builtin_amdgcn_sched_barrier(0);
+            for (int t = 0; t < kPairs; t += 2) {
+                const float4 y = q4[t >> 1];
+                const float d0 = y.x - x[t].x, d1 = y.y - x[t].y;
+                a0 = fmaf(d0, d0, a0);
+                a1 = fmaf(d1, d1, a1);
+                const float d2 = y.z - x[t + 1].x, d3 = y.w - x[t + 1].y;
+                a0 = fmaf(d2, d2, a0);
+                a1 = fmaf(d3, d3, a1);
+                if ((t & 2) == 2) __builtin_amdgcn_sched_barrier(0);
             }
+            __builtin_amdgcn_sched_barrier(0);
         } else {
 #pragma unroll 4
             for (int t = 0; t < groups; ++t) {
                 const float2 x = row[4 * t];
-                const float2 y = qv[4 * t];
+                const float2 y = qv[t];
                 const float d0 = y.x - x.x, d1 = y.y - x.y;
                 a0 = fmaf(d0, d0, a0);
                 a1 = fmaf(d1, d1, a1);

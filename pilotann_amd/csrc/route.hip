@@ -105,15 +105,16 @@ __global__ __launch_bounds__(256) void leaf_dist_kernel(
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
     const int q = blockIdx.x * (blockDim.x / kWave) + wave;
-    float *qv = qv_all + wave * dp;
+    float *qv = qv_all + wave * query_floats(dp);
     if (q < batch)
-        for (int i = lane; i < dp; i += kWave) qv[i] = query[(size_t)q * dp + i];
+        for (int i = lane; i < dp; i += kWave)
+            qv[query_slot(i, dp >> 3)] = query[(size_t)q * dp + i];
     __syncthreads();
     if (q >= batch) return;
     const int64_t group = router ? router[q] : 0;
     const float *leaves = entry_vectors + (size_t)group * n_leaves * dp;
     const int quad = lane >> 2, part = lane & 3;
-    const float2 *qq = reinterpret_cast<const float2 *>(qv) + part;
+    const float2 *qq = reinterpret_cast<const float2 *>(qv) + part * query_run(dp >> 3);
     for (int base = 0; base < n_leaves; base += kRowsPerPass) {
         const int l = base + quad;
         const bool active = l < n_leaves;
@@ -145,7 +146,7 @@ extern "C" int pa_route(int64_t *router, float *dist, const float *query,
     }
     const int waves = 4;
     const unsigned blocks = (unsigned)((batch + waves - 1) / waves);
-    const size_t lds = (size_t)waves * dp * sizeof(float);
+    const size_t lds = (size_t)waves * query_floats(dp) * sizeof(float);
     const int64_t *group = n_routers > 0 ? router : nullptr;
     switch (dp) {
         case 32:

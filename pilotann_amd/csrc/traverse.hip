@@ -385,7 +385,7 @@ __device__ __forceinline__ void eval_rows(const float *__restrict__ storage,
                                           float *cand_key, int n, int dp,
                                           int lane) {
     const int quad = lane >> 2, part = lane & 3;
-    const float2 *qq = reinterpret_cast<const float2 *>(qv) + part;
+    const float2 *qq = reinterpret_cast<const float2 *>(qv) + part * query_run(dp >> 3);
     for (int base = 0; base < n; base += kRowsPerPass) {
         const int c = base + quad;
         const bool active = c < n;
@@ -458,7 +458,7 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
     float *cand_key = reinterpret_cast<float *>(cand_id + kWave);
     float *qv = cand_key + kWave;
     const int dp = DP8 ? DP8 * 8 : a.dp;
-    uint32_t *seen_cache = reinterpret_cast<uint32_t *>(qv + dp);
+    uint32_t *seen_cache = reinterpret_cast<uint32_t *>(qv + query_floats(dp));
     const bool use_cache = a.n_storage <= (0xffff << kSeenCacheLog2);
     const int deg = a.deg;
     uint32_t *seen = a.seen + (size_t)blockIdx.x * (size_t)a.words_per_slot;
@@ -479,7 +479,7 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
         for (int w = lane * 4; w < a.words_per_slot; w += kWave * 4)
             *reinterpret_cast<uint4 *>(seen + w) = make_uint4(0, 0, 0, 0);
         for (int i = lane; i < dp; i += kWave)
-            qv[i] = a.query[(size_t)q * dp + i];
+            qv[query_slot(i, dp >> 3)] = a.query[(size_t)q * dp + i];
         for (int i = lane; i < kSeenCache; i += kWave) seen_cache[i] = 0xffffffffu;
         open.reset(lane);
         Results<S> res;
@@ -814,7 +814,7 @@ int make_plan(int64_t n_storage, int64_t batch, int dp, int ef_total, Plan *p) {
     // final sort of sort_n cells
     const int tail = 2 * p->H + 2 - 256;
     p->lds_cells = tail > p->sort_n ? tail : p->sort_n;
-    p->lds_bytes = p->lds_cells * 8 + kWave * 8 + dp * 4 + kSeenCache * 4;
+    p->lds_bytes = p->lds_cells * 8 + kWave * 8 + query_floats(dp) * 4 + kSeenCache * 4;
 #ifdef PA_EXTRA_LDS  // tuning builds: lower the residency without touching code
     p->lds_bytes += PA_EXTRA_LDS;
 #endif
