@@ -446,19 +446,32 @@ __global__ void reset_work_counter(int *counter) { *counter = 0; }
 
 template <int H, int DP8>
 __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(TraverseArgs a) {
-    extern __shared__ __align__(16) unsigned char smem[];
+    // One static block, in this order: the compiler then knows every LDS
+    // address, and a heap cell [j - 256] is the scalar j * 8 plus a positive
+    // constant that fits the instruction's offset field.
     constexpr int S = (H + kWave - 1) / kWave;
+    constexpr int kSortN = H <= kWave ? kWave : 1 << (floor_log2(H - 1) + 1);
+    constexpr int kHeapCells =
+        OpenList<H>::kLdsCells > kSortN ? OpenList<H>::kLdsCells : kSortN;
+    struct Lds {
+        uint32_t seen_cache[kSeenCache];
+        int cand_id[kWave];
+        float cand_key[kWave];
+        float query[DP8 ? query_floats(8 * DP8) : 4];
+        int2 heap[kHeapCells];  // open list tail; the final sort reuses it
+    };
+    __shared__ __align__(16) Lds lds;
+    extern __shared__ __align__(16) float query_any_length[];  // DP8 == 0 only
     const int lane = threadIdx.x;
-    const int heap_cells = a.lds_cells;
-    float *okey = reinterpret_cast<float *>(smem);
-    int *oval = reinterpret_cast<int *>(okey + heap_cells);
+    float *okey = reinterpret_cast<float *>(lds.heap);
+    int *oval = reinterpret_cast<int *>(okey + kHeapCells);
     OpenList<H> open;
-    open.cells = reinterpret_cast<int2 *>(smem);
-    int *cand_id = oval + heap_cells;
-    float *cand_key = reinterpret_cast<float *>(cand_id + kWave);
-    float *qv = cand_key + kWave;
+    open.cells = lds.heap;
+    int *cand_id = lds.cand_id;
+    float *cand_key = lds.cand_key;
+    float *qv = DP8 ? lds.query : query_any_length;
     const int dp = DP8 ? DP8 * 8 : a.dp;
-    uint32_t *seen_cache = reinterpret_cast<uint32_t *>(qv + query_floats(dp));
+    uint32_t *seen_cache = lds.seen_cache;
     const bool use_cache = a.n_storage <= (0xffff << kSeenCacheLog2);
     const int deg = a.deg;
     uint32_t *seen = a.seen + (size_t)blockIdx.x * (size_t)a.words_per_slot;
@@ -814,7 +827,9 @@ int make_plan(int64_t n_storage, int64_t batch, int dp, int ef_total, Plan *p) {
     // final sort of sort_n cells
     const int tail = 2 * p->H + 2 - 256;
     p->lds_cells = tail > p->sort_n ? tail : p->sort_n;
-    p->lds_bytes = p->lds_cells * 8 + kWave * 8 + query_floats(dp) * 4 + kSeenCache * 4;
+    // dynamic LDS: the query when its length has no specialised kernel (the
+    // rest is static in the kernel)
+    p->lds_bytes = (dp == 32 || dp == 64 || dp == 128) ? 0 : query_floats(dp) * 4;
 #ifdef PA_EXTRA_LDS  // tuning builds: lower the residency without touching code
     p->lds_bytes += PA_EXTRA_LDS;
 #endif
