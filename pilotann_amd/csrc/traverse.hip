@@ -435,13 +435,19 @@ __global__ void reset_work_counter(int *counter) { *counter = 0; }
 #define PA_TIMER(i) do {} while (0)
 #endif
 
-// Up to H = 256 the kernel fits the register budget of five wavefronts per
-// SIMD (96 VGPRs), which measures faster than four; larger result lists need
-// more registers and are left to the compiler.
+// Wavefronts per SIMD the register allocator must fit.  A budget a few
+// registers under what the code needs costs more (spills, serialised loads)
+// than the extra wavefront brings — measured: H = 256 with 128-float rows
+// needs 113 registers and is 4 % faster at four wavefronts (128) than squeezed
+// into the 96 of five, while three wavefronts are 11 % slower than four.  So
+// only a floor is given, under which no instance has to be squeezed (the
+// largest heaps are bounded by their LDS anyway), and the allocator's own
+// count decides the residency above it: 8 for the smallest instances, 4 for
+// H = 256 with 128-float rows.
 #ifdef PA_WAVES_PER_EU
 #define PA_OCCUPANCY(H) __attribute__((amdgpu_waves_per_eu(PA_WAVES_PER_EU, PA_WAVES_PER_EU)))
 #else
-#define PA_OCCUPANCY(H) __attribute__((amdgpu_waves_per_eu((H) <= 256 ? 5 : 1, (H) <= 256 ? 5 : 8)))
+#define PA_OCCUPANCY(H) __attribute__((amdgpu_waves_per_eu((H) <= 512 ? 4 : (H) <= 1024 ? 2 : 1, 8)))
 #endif
 
 template <int H, int DP8>
@@ -858,6 +864,12 @@ int make_plan(int64_t n_storage, int64_t batch, int dp, int ef_total, Plan *p) {
         cus = it->second.first, per_cu = it->second.second;
     }
     if (per_cu < 1) per_cu = 1;
+    // more than five wavefronts per SIMD have measured slower on every
+    // instance that fits them (the SIMDs' issue slots are the bound)
+#ifndef PA_MAX_WAVES_PER_CU
+#define PA_MAX_WAVES_PER_CU 20
+#endif
+    if (per_cu > PA_MAX_WAVES_PER_CU) per_cu = PA_MAX_WAVES_PER_CU;
     int64_t slots = (int64_t)per_cu * cus;
     if (slots < 1) slots = 1;
     if (slots > batch) slots = batch;
