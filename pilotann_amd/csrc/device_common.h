@@ -136,13 +136,20 @@ __device__ __forceinline__ float quad_square_dist(const float2 *row,
         }
     }
     // accumulators 0..7 left to right: lane 0 has (0, 1), lane 1 (2, 3), ...
-    float s = a0 + a1;
-    s += dpp_f<0x55, 0xF>(a0);  // quad_perm [1,1,1,1]
-    s += dpp_f<0x55, 0xF>(a1);
-    s += dpp_f<0xAA, 0xF>(a0);  // quad_perm [2,2,2,2]
-    s += dpp_f<0xAA, 0xF>(a1);
-    s += dpp_f<0xFF, 0xF>(a0);  // quad_perm [3,3,3,3]
-    s += dpp_f<0xFF, 0xF>(a1);
+    // One v_add_f32_dpp per term (the other lanes' accumulators come in as the
+    // swizzled operand); the s_nop covers the two wait states a DPP read needs
+    // after the last FMA wrote a0 / a1.
+    float s;
+    asm("s_nop 1\n\t"
+        "v_add_f32 %0, %1, %2\n\t"
+        "v_add_f32_dpp %0, %1, %0 quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf\n\t"
+        "v_add_f32_dpp %0, %2, %0 quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf\n\t"
+        "v_add_f32_dpp %0, %1, %0 quad_perm:[2,2,2,2] row_mask:0xf bank_mask:0xf\n\t"
+        "v_add_f32_dpp %0, %2, %0 quad_perm:[2,2,2,2] row_mask:0xf bank_mask:0xf\n\t"
+        "v_add_f32_dpp %0, %1, %0 quad_perm:[3,3,3,3] row_mask:0xf bank_mask:0xf\n\t"
+        "v_add_f32_dpp %0, %2, %0 quad_perm:[3,3,3,3] row_mask:0xf bank_mask:0xf"
+        : "=&v"(s)
+        : "v"(a0), "v"(a1));
     return s;
 }
 
