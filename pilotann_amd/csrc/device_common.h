@@ -55,6 +55,7 @@ __device__ __forceinline__ float wave_max(float x) {
 // that each step is one instruction; the s_nop covers the two wait states a
 // DPP read needs after a vector write of the same register.
 __device__ __forceinline__ int wave_max_key(int x) {
+#ifdef PA_WAVE_MAX_ASM
     asm("s_nop 1\n\t"
         "v_max_i32_dpp %0, %0, %0 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
         "s_nop 1\n\t"
@@ -69,6 +70,15 @@ __device__ __forceinline__ int wave_max_key(int x) {
         "v_max_i32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
         "s_nop 1"
         : "+v"(x));
+#else
+    constexpr int kLow = (int)0x80000000;
+    x = max(x, __builtin_amdgcn_update_dpp(kLow, x, 0xB1, 0xF, 0xF, false));
+    x = max(x, __builtin_amdgcn_update_dpp(kLow, x, 0x4E, 0xF, 0xF, false));
+    x = max(x, __builtin_amdgcn_update_dpp(kLow, x, 0x141, 0xF, 0xF, false));
+    x = max(x, __builtin_amdgcn_update_dpp(kLow, x, 0x140, 0xF, 0xF, false));
+    x = max(x, __builtin_amdgcn_update_dpp(kLow, x, 0x142, 0xA, 0xF, false));
+    x = max(x, __builtin_amdgcn_update_dpp(kLow, x, 0x143, 0xC, 0xF, false));
+#endif
     return __builtin_amdgcn_readlane(x, kWave - 1);
 }
 
