@@ -20,6 +20,8 @@ def router_init(storage: torch.Tensor, init_nodes: list, n_routers: int,
     n_storage = storage.size(0)
     init_nodes = list(init_nodes) if init_nodes else []
 
+    if n_routers > n_storage:
+        raise RuntimeError(f'{n_routers} routes from {n_storage} nodes')
     chosen = [rng.randrange(n_storage)]
     member = set(chosen)
     while len(chosen) < n_routers:
@@ -34,6 +36,11 @@ def router_init(storage: torch.Tensor, init_nodes: list, n_routers: int,
     visited = set()
     entry_nodes = [[] for _ in range(n_routers)]
     per_round = min(1024, n_routers ** 2)
+    if n_routers > n_storage or per_round * n_leaves > n_storage:
+        # the rounds below draw unseen nodes until they have enough
+        raise RuntimeError(
+            f'router{n_routers}x{n_leaves} needs {per_round * n_leaves} '
+            f'distinct nodes, the set has {n_storage}')
     for _ in range(n_leaves):
         nodes = []
         while len(nodes) < per_round:

@@ -1,6 +1,7 @@
 """Build-time helpers: formats the search path relies on and the properties
 the reference's tests state for them (test/kernel/test_routing.py:6-33,
 test_svd.py, test_graphs.py)."""
+import pytest
 import torch
 
 from pilotann_amd import utils
@@ -91,3 +92,9 @@ def test_recall():
     a = torch.tensor([[1, 2, 3], [4, 5, 6]])
     b = torch.tensor([[3, 2, 9], [7, 8, 9]])
     assert abs(utils.recall(a, b) - (2 / 3 + 0) / 2) < 1e-9
+
+
+def test_router_init_rejects_a_set_too_small_for_it():
+    x = torch.rand(500, 16)
+    with pytest.raises(RuntimeError):
+        utils.router_init(x, None, 32, 32, seed=1)   # needs 1024 * 32 nodes
