@@ -326,52 +326,59 @@ struct OpenList {
     }
 };
 
-// ---- result list: the H smallest distances, S entries per lane --------------
+// ---- result list: the H smallest distances ------------------------------------
 //
 // The reference keeps them in a heap of negated keys whose root is the worst
 // kept (traverse_cpu.cpp:21-39): a candidate enters iff its distance is
 // strictly below that root, and replaces it.  Which array cell holds what has
-// no effect on the search; only the set and its maximum do.  Empty cells hold
-// +inf (so the maximum is +inf until H candidates came), cells beyond H hold
-// -inf and never win.
+// no effect on the search; only the set and its maximum do.  Here the cells
+// are a flat LDS array, S per lane (lane l owns cells l*S .. l*S+S-1), of which
+// the registers keep only each lane's maximum, the wavefront's maximum and the
+// position of one cell that holds it: an insert is one store to that cell,
+// one read of every lane's own cells and a wavefront maximum.  Empty cells
+// hold +inf (so the maximum is +inf until H candidates came), cells beyond H
+// hold -inf and never win.
 
 template <int S>
 struct Results {
     static constexpr int kInf = 0x7f800000;      // float_to_key(+inf)
     static constexpr int kNegInf = (int)0x807fffff;  // float_to_key(-inf)
-    int key[S];   // float_to_key of the distance
-    int val[S];
+    int *rk;      // float_to_key of the distance, kWave * S cells
+    int *rv;
     int lane_max;
     int worst;    // uniform
+    int pos;      // uniform: a cell whose key is `worst`
 
     __device__ __forceinline__ void init(int H, int lane) {
         lane_max = kNegInf;
 #pragma unroll
         for (int s = 0; s < S; ++s) {
-            key[s] = (s * kWave + lane < H) ? kInf : kNegInf;
-            val[s] = -1;
-            lane_max = max(lane_max, key[s]);
+            const int c = lane * S + s;
+            const int k = c < H ? kInf : kNegInf;
+            rk[c] = k, rv[c] = -1;
+            lane_max = max(lane_max, k);
         }
         worst = kInf;
+        pos = 0;
     }
-    // Caller has checked k < worst.  The first lane whose maximum is the
-    // worst replaces its first cell that holds it (branch-free: every lane
-    // runs the same selects).
+    // Caller has checked k < worst.
     __device__ __forceinline__ void insert(int k, int v, int lane) {
-        const unsigned long long holders = __ballot(lane_max == worst);
-        const bool mine = lane == __builtin_ctzll(holders);
-        bool open = mine;
-        int m = kNegInf;
+        rk[pos] = k, rv[pos] = v;  // every lane, the same cell
+        wave_sync();
+        int key[S];
 #pragma unroll
-        for (int s = 0; s < S; ++s) {
-            const bool hit = open && key[s] == worst;
-            key[s] = hit ? k : key[s];
-            val[s] = hit ? v : val[s];
-            open = open && !hit;
-            m = max(m, key[s]);
-        }
+        for (int s = 0; s < S; ++s) key[s] = rk[lane * S + s];
+        int m = key[0];
+#pragma unroll
+        for (int s = 1; s < S; ++s) m = max(m, key[s]);
         lane_max = m;
         worst = wave_max_key(lane_max);
+        // the first lane that holds the new maximum, its first such cell
+        const int holder = __builtin_ctzll(__ballot(lane_max == worst));
+        int c = lane * S + S - 1;
+#pragma unroll
+        for (int s = S - 2; s >= 0; --s) c = key[s] == worst ? lane * S + s : c;
+        pos = __builtin_amdgcn_readlane(c, holder);
     }
 };
 
@@ -447,7 +454,7 @@ __global__ void reset_work_counter(int *counter) { *counter = 0; }
 #ifdef PA_WAVES_PER_EU
 #define PA_OCCUPANCY(H) __attribute__((amdgpu_waves_per_eu(PA_WAVES_PER_EU, PA_WAVES_PER_EU)))
 #else
-#define PA_OCCUPANCY(H) __attribute__((amdgpu_waves_per_eu((H) <= 512 ? 4 : (H) <= 1024 ? 2 : 1, 8)))
+#define PA_OCCUPANCY(H) __attribute__((amdgpu_waves_per_eu((H) <= 256 ? 4 : (H) <= 384 ? 3 : (H) <= 1024 ? 2 : 1, 8)))
 #endif
 
 template <int H, int DP8>
@@ -465,6 +472,8 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
         float cand_key[kWave];
         float query[DP8 ? query_floats(8 * DP8) : 4];
         int2 heap[kHeapCells];  // open list tail; the final sort reuses it
+        int res_key[S * kWave];  // result list
+        int res_val[S * kWave];
     };
     __shared__ __align__(16) Lds lds;
     extern __shared__ __align__(16) float query_any_length[];  // DP8 == 0 only
@@ -502,6 +511,7 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
         for (int i = lane; i < kSeenCache; i += kWave) seen_cache[i] = 0xffffffffu;
         open.reset(lane);
         Results<S> res;
+        res.rk = lds.res_key, res.rv = lds.res_val;
         res.init(H, lane);
         __threadfence();
         wave_sync();
@@ -633,9 +643,13 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
 
         // traverse_cpu.cpp:138-148: storage rows -> global ids, then the
         // entries compete for a result slot.
+        wave_sync();
 #pragma unroll
-        for (int s = 0; s < S; ++s)
-            if (res.val[s] >= 0) res.val[s] = a.gid[res.val[s]];
+        for (int s = 0; s < S; ++s) {
+            const int row = res.rv[lane * S + s];
+            if (row >= 0) res.rv[lane * S + s] = a.gid[row];
+        }
+        wave_sync();
         for (int base = 0; base < a.n_init; base += kWave) {
             const int i = base + lane;
             int u = -1;
@@ -664,8 +678,8 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
         wave_sync();
 #pragma unroll
         for (int s = 0; s < S; ++s) {
-            const int e = s * kWave + lane;
-            if (e < H) okey[e] = key_to_float(res.key[s]), oval[e] = res.val[s];
+            const int e = lane * S + s;
+            if (e < H) okey[e] = key_to_float(res.rk[e]), oval[e] = res.rv[e];
         }
         wave_sync();
         for (int size = 2; size <= a.sort_n; size <<= 1) {
