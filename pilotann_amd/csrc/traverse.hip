@@ -58,7 +58,9 @@ constexpr int kSeenCache = 1 << kSeenCacheLog2;  // LDS words remembering visite
 // integers (float_to_key) so that every comparison of a walk is a scalar
 // integer compare.  All lanes run the same, uniform, control flow; the walks
 // are unrolled by level so that each level is a dozen instructions.  After
-// each operation the heap is, cell for cell, the reference's.
+// each operation the heap is, cell for cell, the reference's.  Every lane
+// stores the same values to the same LDS cells and reads the same cells, so a
+// lane only ever reads back its own stores and the walks need no fences.
 __device__ __forceinline__ int float_to_key(float x) {
     const int b = __float_as_int(x);
     return b ^ ((b >> 31) & 0x7fffffff);
@@ -245,7 +247,6 @@ struct OpenList {
         for (int L = 1; L <= kDepth; ++L) {
             if (L == kDepth && 2 * j > kSize) {
                 put(kind(L - 1), j, kInf, -1, lane);
-                wave_sync();
                 return;
             }
             int c, ck, cv;
@@ -264,13 +265,18 @@ struct OpenList {
             j = c;
         }
         put(kind(kDepth), j, kInf, -1, lane);
-        wave_sync();
     }
 
     // heapq.cuh:47-77: walk to a leaf through the larger child (left on
     // ties), overwrite it when the new key is strictly smaller, let the new
-    // entry rise.
-    __device__ __forceinline__ void replace(int k, int v, int lane) {
+    // entry rise.  In two parts so that the caller can put independent work
+    // between them: the walk is straight-line code, the rise branches.
+    struct Leaf {
+        int j;       // the leaf
+        int key;     // its key
+        bool bottom; // it is on level kDepth
+    };
+    __device__ __forceinline__ Leaf walk_to_large_leaf() const {
         const Choice ch = choices<true>();
         int j = 1;
         bool bottom = true;  // the walk reached level kDepth
@@ -293,12 +299,18 @@ struct OpenList {
             }
         }
         // the leaf's key: the walk has it already when the leaf is in LDS
-        int leaf_key;
+        Leaf leaf;
+        leaf.j = j, leaf.bottom = bottom;
         if (bottom)
-            leaf_key = kind(kDepth) == 3 ? walked_key : key_of(kind(kDepth), j);
+            leaf.key = kind(kDepth) == 3 ? walked_key : key_of(kind(kDepth), j);
         else
-            leaf_key = kind(kDepth - 1) == 3 ? walked_key : key_of(kind(kDepth - 1), j);
-        if (k >= leaf_key) return;
+            leaf.key = kind(kDepth - 1) == 3 ? walked_key : key_of(kind(kDepth - 1), j);
+        return leaf;
+    }
+    __device__ __forceinline__ void replace_leaf(const Leaf &leaf, int k, int v,
+                                                 int lane) {
+        if (k >= leaf.key) return;
+        int j = leaf.j;
         // one store per level: the parent's entry while it is larger than
         // the new key, the new entry where the rise stops
         auto rise = [&](const int L) -> bool {
@@ -310,19 +322,15 @@ struct OpenList {
             j = up;
             return stop;
         };
-        if (bottom && rise(kDepth)) {
-            wave_sync();
-            return;
-        }
+        if (leaf.bottom && rise(kDepth)) return;
 #pragma unroll
-        for (int L = kDepth - 1; L >= 1; --L) {
-            if (rise(L)) {
-                wave_sync();
-                return;
-            }
-        }
+        for (int L = kDepth - 1; L >= 1; --L)
+            if (rise(L)) return;
         put(0, 1, k, v, lane);
-        wave_sync();
+    }
+    __device__ __forceinline__ void replace(int k, int v, int lane) {
+        const Leaf leaf = walk_to_large_leaf();
+        replace_leaf(leaf, k, v, lane);
     }
 };
 
@@ -361,13 +369,16 @@ struct Results {
         worst = kInf;
         pos = 0;
     }
-    // Caller has checked k < worst.
-    __device__ __forceinline__ void insert(int k, int v, int lane) {
-        rk[pos] = k, rv[pos] = v;  // every lane, the same cell
-        wave_sync();
-        int key[S];
+    // Caller has checked k < worst.  In two parts so that the caller can put
+    // independent work between the LDS traffic and its use.
+    __device__ __forceinline__ void begin_insert(int k, int v, int lane, int (&key)[S]) {
+        // Every lane stores the same pair to the same cell, so the lane that
+        // owns the cell reads back its own store: program order is enough.
+        rk[pos] = k, rv[pos] = v;
 #pragma unroll
         for (int s = 0; s < S; ++s) key[s] = rk[lane * S + s];
+    }
+    __device__ __forceinline__ void finish_insert(int lane, const int (&key)[S]) {
         int m = key[0];
 #pragma unroll
         for (int s = 1; s < S; ++s) m = max(m, key[s]);
@@ -379,6 +390,11 @@ struct Results {
 #pragma unroll
         for (int s = S - 2; s >= 0; --s) c = key[s] == worst ? lane * S + s : c;
         pos = __builtin_amdgcn_readlane(c, holder);
+    }
+    __device__ __forceinline__ void insert(int k, int v, int lane) {
+        int key[S];
+        begin_insert(k, v, lane, key);
+        finish_insert(lane, key);
     }
 };
 
@@ -628,8 +644,11 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
                         const int dj = __builtin_amdgcn_readlane(d, j);
                         if (dj >= res.worst) continue;
                         const int vj = __builtin_amdgcn_readlane(id, j);
-                        res.insert(dj, vj, lane);
-                        open.replace(dj, vj, lane);
+                        int mine[S];
+                        res.begin_insert(dj, vj, lane, mine);
+                        const typename OpenList<H>::Leaf leaf = open.walk_to_large_leaf();
+                        res.finish_insert(lane, mine);
+                        open.replace_leaf(leaf, dj, vj, lane);
                         n_admit += 1;
                     }
                     PA_TIMER(4);
