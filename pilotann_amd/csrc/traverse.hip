@@ -221,13 +221,31 @@ struct OpenList {
         return ch;
     }
     // the child of j the walk takes on register level L (1..7), L < kDepth
-    // or the pair is known to be complete
+    // or the pair is known to be complete: 2j + (bit of the pair in the
+    // level's mask), three scalar instructions.  s_bitcmp1_b64 looks at the
+    // low six bits of its index only, so node numbers serve as lane numbers
+    // (bank B holds node j in lane j - 64, banks C/D the children of node j
+    // in lane j - 64).
     __device__ __forceinline__ int step_down(const int L, int j,
                                              const Choice &ch) const {
-        const int c = 2 * j;
-        if (kind(L) == 0) return add_if_bit(c, ch.a, c + 1);
-        if (kind(L) == 1) return add_if_bit(c, ch.b, c + 1 - 64);
-        return add_if_bit(c, ch.cd, j - 64);
+        int r;
+        if (kind(L) <= 1) {
+            // t = 2j + 1, the right child, whose lane holds the pair's bit
+            asm("s_lshl1_add_u32 %0, %1, 1\n\t"
+                "s_bitcmp1_b64 %2, %0\n\t"
+                "s_addc_u32 %0, %0, -1"
+                : "=&s"(r)
+                : "s"(j), "s"(kind(L) == 0 ? ch.a : ch.b)
+                : "scc");
+        } else {
+            asm("s_lshl_b32 %0, %1, 1\n\t"
+                "s_bitcmp1_b64 %2, %1\n\t"
+                "s_addc_u32 %0, %0, 0"
+                : "=&s"(r)
+                : "s"(j), "s"(ch.cd)
+                : "scc");
+        }
+        return r;
     }
 
     // heapq.cuh:37-45 with the sift of :13-29: the root leaves, (inf, -1)
