@@ -260,26 +260,51 @@ struct OpenList {
         out_k = rl(Ak, 1);
         out_v = rl(Av, 1);
         const Choice ch = choices<false>();
-        int j = 1;
+        // Register levels in three passes, so that no read waits for a write
+        // of the same bank: the path (masks only), then every entry on it,
+        // then the stores.  Reading first is the same thing: a level's store
+        // goes to the cell above the one read.
+        constexpr int kRegLevels = kDepth < 7 ? kDepth : 7;
+        int node[kRegLevels + 1];
+        node[0] = 1;
+        bool cut = false;  // level kDepth has no node below node[kDepth - 1]
 #pragma unroll
-        for (int L = 1; L <= kDepth; ++L) {
+        for (int L = 1; L <= kRegLevels; ++L) {
+            if (L == kDepth && 2 * node[L - 1] > kSize) {
+                cut = true;
+                node[L] = node[L - 1];
+            } else {
+                node[L] = step_down(L, node[L - 1], ch);
+            }
+        }
+        int ck[kRegLevels + 1], cv[kRegLevels + 1];
+#pragma unroll
+        for (int L = 1; L <= kRegLevels; ++L) {
+            ck[L] = key_of(kind(L), node[L]);
+            cv[L] = val_of(kind(L), node[L]);
+        }
+#pragma unroll
+        for (int L = 1; L <= kRegLevels; ++L) {
+            if (L == kDepth && cut) {
+                put(kind(L - 1), node[L - 1], kInf, -1, lane);
+                return;
+            }
+            put(kind(L - 1), node[L - 1], ck[L], cv[L], lane);
+        }
+        int j = node[kRegLevels];
+#pragma unroll
+        for (int L = kRegLevels + 1; L <= kDepth; ++L) {
             if (L == kDepth && 2 * j > kSize) {
                 put(kind(L - 1), j, kInf, -1, lane);
                 return;
             }
-            int c, ck, cv;
-            if (kind(L) <= 2) {
-                c = step_down(L, j, ch);
-                ck = key_of(kind(L), c), cv = val_of(kind(L), c);
-            } else {
-                int ka, kb, va, vb;
-                pair(3, true, 2 * j, ka, kb, va, vb);
-                if (L == kDepth) kb = 2 * j == kSize ? ka : kb;
-                ck = min(ka, kb);
-                cv = ck != ka ? vb : va;
-                c = add_if_ne(2 * j, ck, ka);
-            }
-            put(kind(L - 1), j, ck, cv, lane);
+            int ka, kb, va, vb;
+            pair(3, true, 2 * j, ka, kb, va, vb);
+            if (L == kDepth) kb = 2 * j == kSize ? ka : kb;
+            const int k = min(ka, kb);
+            const int v = k != ka ? vb : va;
+            const int c = add_if_ne(2 * j, k, ka);
+            put(kind(L - 1), j, k, v, lane);
             j = c;
         }
         put(kind(kDepth), j, kInf, -1, lane);
