@@ -30,12 +30,12 @@ METRIC = 'QPS @ recall@10>=0.90 (1M x 768 fp32, 1 GPU); traversal HBM GB/s'
 HBM_PEAK_GBS = 8000.0
 
 CONFIGS = {
-    # BASELINE.json configs[2]: the configuration the metric is quoted on
+    # the configuration the metric is quoted on
     'c3': dict(n=1_000_000, d=768, dp=128, n_centers=1024, sigma=1.0,
                decay=0.5, normalize=True, ratio=0.25, graph='nsw64',
                entry='router64x64', queries=10_000, k=10,
                ef_sweep=[4, 8, 16, 24, 32, 48, 64], seed=301),
-    # BASELINE.json configs[1]
+    # the smaller 96-dimensional configuration
     'c2': dict(n=1_000_000, d=96, dp=64, n_centers=256, sigma=1.0,
                decay=0.5, normalize=False, ratio=0.25, graph='nsw32',
                entry='router32x32', queries=10_000, k=10,
