@@ -350,6 +350,11 @@ struct OpenList {
             leaf.key = kind(kDepth - 1) == 3 ? walked_key : key_of(kind(kDepth - 1), j);
         return leaf;
     }
+    // SPARSE: the heap is nearly empty (the entries of a query are pushed),
+    // so most ancestors of the leaf are (inf, -1), and so is everything below
+    // such an ancestor: moving it down would write (inf, -1) over (inf, -1)
+    // and is left out.
+    template <bool SPARSE = false>
     __device__ __forceinline__ void replace_leaf(const Leaf &leaf, int k, int v,
                                                  int lane) {
         if (k >= leaf.key) return;
@@ -359,6 +364,10 @@ struct OpenList {
         auto rise = [&](const int L) -> bool {
             const int up = j >> 1;
             const int pk = key_of(kind(L - 1), up);
+            if (SPARSE && pk == kInf) {
+                j = up;
+                return false;
+            }
             const int pv = val_of(kind(L - 1), up);
             const bool stop = pk <= k;
             put(kind(L), j, stop ? k : pk, stop ? v : pv, lane);
@@ -371,9 +380,10 @@ struct OpenList {
             if (rise(L)) return;
         put(0, 1, k, v, lane);
     }
+    template <bool SPARSE = false>
     __device__ __forceinline__ void replace(int k, int v, int lane) {
         const Leaf leaf = walk_to_large_leaf();
-        replace_leaf(leaf, k, v, lane);
+        replace_leaf<SPARSE>(leaf, k, v, lane);
     }
 };
 
@@ -572,7 +582,12 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
         Results<S> res;
         res.rk = lds.res_key, res.rv = lds.res_val;
         res.init(H, lane);
-        __threadfence();
+        // The clearing stores must have reached the cache level where the
+        // atomic ORs are performed before the first OR is issued.  Only this
+        // wavefront touches the slice, so waiting for its own stores is
+        // enough; a device-scope fence here would write back and invalidate
+        // caches once per query.
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         wave_sync();
 
         // traverse_cpu.cpp:69-79: entries are marked and pushed on the open
@@ -602,7 +617,7 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
                 const int rj = __builtin_amdgcn_readlane(row, j);
                 const float dj =
                     __int_as_float(__builtin_amdgcn_readlane(__float_as_int(d), j));
-                open.replace(float_to_key(dj), rj >= 0 ? rj : -2 - (base + j), lane);
+                open.template replace<true>(float_to_key(dj), rj >= 0 ? rj : -2 - (base + j), lane);
             }
         }
 
