@@ -95,11 +95,20 @@ class IndexStaged(nn.Module):
         search form of the subgraph is prepared here, once."""
         self.cuda_device = device
         self.entry.to(device=device)
-        self.mapping_cuda = self.mapping.to(device=device)
         self.subgraph_cuda = GraphModule(self.subgraph.indptr,
                                          self.subgraph.indices).to(device)
         rows = torch.index_select(self.storage, 0, self.nodelist)
-        self.storage_cuda = rows[:, :self.d_principle].contiguous().to(device)
+        rows = rows[:, :self.d_principle].contiguous().to(device)
+        # device rows in a locality-preserving order (utils/layout.py); the
+        # host copies (checkpoint format) keep the order of the global ids
+        order = utils.locality_order(rows, seed=self.seed)
+        place = torch.empty_like(order)
+        place[order] = torch.arange(order.numel(), device=order.device)
+        self.storage_cuda = rows[order].contiguous()
+        mapping = self.mapping.to(device=device).clone()
+        sampled = mapping >= 0
+        mapping[sampled] = place[mapping[sampled]]
+        self.mapping_cuda = mapping
         if torch.device(device).type == 'cuda':
             kernels.prepare_graph(
                 self.subgraph_cuda.indptr, self.subgraph_cuda.indices,

@@ -13,8 +13,10 @@ from .svd import svd
 from .graphs import knn_graph, graph_init, subgraph_init, graph_sampling
 from .router import router_init
 from .synth import gaussian_mixture, brute_force_topk
+from .layout import locality_order
 
 __all__ = [
     'recall', 'svd', 'knn_graph', 'graph_init', 'subgraph_init',
     'graph_sampling', 'router_init', 'gaussian_mixture', 'brute_force_topk',
+    'locality_order',
 ]

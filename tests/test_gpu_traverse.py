@@ -203,3 +203,30 @@ def test_degree_one_chain(device):
                           torch.full((1, 1), float((n + 10) ** 2), device=device), 1)
     cap = 2 * 4 * ef
     assert out_I.flatten().tolist() == [cap - i for i in range(4 * ef)]
+
+
+def test_row_order_does_not_change_results(device):
+    """The storage rows may be laid out in any order (``mapping`` says which
+    row a node has): same ids, same distances, bit for bit."""
+    p = Problem(n=6000, d=64, deg=32, sample_ratio=0.5, seed=31, n_query=80)
+    init_I, init_D = p.entries(32, seed=9, dp=64)
+    I_a, D_a, _ = run_gpu(p, 64, 32, init_I, init_D, device)
+    from pilotann_amd import utils
+    rows = p.x[p.nodelist]
+    for order in (torch.randperm(rows.size(0), generator=torch.Generator().manual_seed(1)),
+                  utils.locality_order(rows, seed=2)):
+        place = torch.empty_like(order)
+        place[order] = torch.arange(order.numel())
+        mapping = p.mapping.clone()
+        mapping[p.mapping >= 0] = place[p.mapping[p.mapping >= 0]]
+        out_I = torch.empty(80, 4, 32, dtype=torch.long, device=device)
+        out_D = torch.empty(80, 4, 32, dtype=torch.float, device=device)
+        kernels.traverse_cuda(
+            output_I=out_I, output_D=out_D, indptr=p.sub_indptr.to(device),
+            indices=p.sub_indices.to(device), mapping=mapping.to(device),
+            storage=rows[order].contiguous().to(device),
+            query=p.query.contiguous().to(device), initial_I=init_I.to(device),
+            initial_D=init_D.to(device), n_neighbors=p.deg)
+        torch.cuda.synchronize()
+        assert np.array_equal(out_I.flatten(1).cpu().numpy(), I_a)
+        assert np.array_equal(out_D.flatten(1).cpu().numpy(), D_a)

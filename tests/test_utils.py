@@ -98,3 +98,17 @@ def test_router_init_rejects_a_set_too_small_for_it():
     x = torch.rand(500, 16)
     with pytest.raises(RuntimeError):
         utils.router_init(x, None, 32, 32, seed=1)   # needs 1024 * 32 nodes
+
+
+def test_locality_order_is_a_permutation_that_groups_neighbours():
+    x = utils.gaussian_mixture(6000, 16, 24, 0.2, seed=4)
+    order = utils.locality_order(x, n_cells=24, seed=1)
+    assert sorted(order.tolist()) == list(range(6000))
+    assert torch.equal(order, utils.locality_order(x, n_cells=24, seed=1))
+    # rows next to each other in the new order are far closer than rows next
+    # to each other in the old one
+    y = x[order]
+    new_gap = (y[1:] - y[:-1]).norm(dim=1).mean()
+    old_gap = (x[1:] - x[:-1]).norm(dim=1).mean()
+    assert new_gap < 0.5 * old_gap
+    assert utils.locality_order(x[:5]).numel() == 5
