@@ -34,7 +34,7 @@ enum {
     PA_E_DIM = -3,         /* vector length not a multiple of 8 (distance.h:35-36) */
     PA_E_NEIGHBORS = -4,   /* n_neighbors outside 1..64                          */
     PA_E_EF = -5,          /* beam * ef outside 1..2048                          */
-    PA_E_WORKSPACE = -6,   /* workspace smaller than pa_traverse_plan() asked    */
+    PA_E_WORKSPACE = -6,   /* workspace too small or not 256-byte aligned          */
     PA_E_GRAPH = -7,       /* pa_graph_prepare found a malformed graph           */
     PA_E_LEAVES = -8,      /* n_leaves not a multiple of 32 (routing_cuda.cu:90) */
     PA_E_CHUNK = -9,       /* batch not a multiple of chunk (pipeline_cpu.cpp:58) */

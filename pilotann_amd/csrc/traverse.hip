@@ -991,7 +991,7 @@ extern "C" const char *pa_error_string(int code) {
         case PA_E_DIM: return "vector length must be a multiple of 8";
         case PA_E_NEIGHBORS: return "n_neighbors must be in 1..64";
         case PA_E_EF: return "beam * ef must be in 1..2048";
-        case PA_E_WORKSPACE: return "workspace too small";
+        case PA_E_WORKSPACE: return "workspace too small or not 256-byte aligned";
         case PA_E_GRAPH: return "malformed graph (see status word)";
         case PA_E_LEAVES: return "n_leaves must be a multiple of 32";
         case PA_E_CHUNK: return "batch must be a multiple of chunk_size";
@@ -1063,6 +1063,7 @@ extern "C" int pa_traverse(int64_t *out_I, float *out_D, const int32_t *adj,
         !workspace || (n_init > 0 && (!init_I || !init_D)))
         return PA_E_NULL;
     if (workspace_bytes < p.workspace_bytes) return PA_E_WORKSPACE;
+    if (reinterpret_cast<uintptr_t>(workspace) % 256) return PA_E_WORKSPACE;
 
     TraverseArgs a;
     a.out_I = out_I, a.out_D = out_D;
