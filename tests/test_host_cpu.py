@@ -63,6 +63,39 @@ def test_traverse_refine_equals_oracle(problem, ef, dp, n_init):
     assert np.array_equal(hI.numpy(), ref[2]) and np.array_equal(hD.numpy(), ref[3])
 
 
+def test_long_rows():
+    """Rows of 400 floats (the small cases have 64): host stages bit-identical
+    to the oracle."""
+    p = Problem(n=3000, d=400, n_centers=12, deg=32, sample_ratio=0.5, seed=17,
+                n_query=60)
+    B, k, ef, dp, n_init = 60, 10, 24, 32, 64
+    init_I, init_D = p.entries(32, seed=3)
+    out_I = torch.empty(B, k, dtype=torch.long)
+    out_D = torch.empty(B, k)
+    kernels.traverse_cpu(out_I, out_D, init_I.clone(), init_D.clone(),
+                         p.indptr, p.indices, p.x, p.query, ef)
+    ref_I = np.empty((B, k), np.int64)
+    ref_D = np.empty((B, k), np.float32)
+    oracle.traverse_cpu(ref_I, ref_D, init_I.numpy().copy(), init_D.numpy().copy(),
+                        p.indptr.numpy(), p.indices.numpy(), p.x.numpy(),
+                        p.query.numpy(), ef)
+    assert np.array_equal(out_I.numpy(), ref_I) and np.array_equal(out_D.numpy(), ref_D)
+    init_I, init_D = p.entries(n_init, seed=4, dp=dp, sampled_only=True)
+    sub, full = [p.sub_indptr, p.sub_indices], [p.indptr, p.indices]
+    out = [torch.empty(B, k, dtype=torch.long), torch.empty(B, k),
+           torch.empty(B, n_init, dtype=torch.long), torch.empty(B, n_init)]
+    kernels.traverse_refine(out[0], out[1], out[2], out[3], init_I.clone(),
+                            init_D.clone(), sub, full, p.x, p.query, ef, dp)
+    ref = [np.empty((B, k), np.int64), np.empty((B, k), np.float32),
+           np.empty((B, n_init), np.int64), np.empty((B, n_init), np.float32)]
+    oracle.traverse_refine(ref[0], ref[1], ref[2], ref[3], init_I.numpy().copy(),
+                           init_D.numpy().copy(), [g.numpy() for g in sub],
+                           [g.numpy() for g in full], p.x.numpy(),
+                           p.query.numpy(), ef, dp)
+    for a, b in zip(out, ref):
+        assert np.array_equal(a.numpy(), b)
+
+
 def test_host_argument_errors(problem):
     p = problem
     B = p.query.size(0)
