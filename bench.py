@@ -35,6 +35,11 @@ CONFIGS = {
                decay=0.5, normalize=True, ratio=0.25, graph='nsw64',
                entry='router64x64', queries=10_000, k=10,
                ef_sweep=[4, 8, 16, 24, 32, 48, 64], seed=301),
+    # large result lists: top-100, ef 256 / 512 (heaps of 1024 / 2048 entries)
+    'c4': dict(n=1_000_000, d=768, dp=128, n_centers=1024, sigma=1.0,
+               decay=0.5, normalize=True, ratio=0.5, graph='nsw64',
+               entry='router64x64', queries=10_000, k=100,
+               ef_sweep=[256, 512], seed=301),
     # the smaller 96-dimensional configuration
     'c2': dict(n=1_000_000, d=96, dp=64, n_centers=256, sigma=1.0,
                decay=0.5, normalize=False, ratio=0.25, graph='nsw32',
@@ -299,7 +304,7 @@ def main():
                         f'{cfg["n_centers"]}-component mixture, dp={dp}, '
                         f'sample_ratio={cfg["ratio"]}, {cfg["graph"]}, '
                         f'{cfg["entry"]}, {B} queries, top-{k}',
-            'ef': ef, 'recall_at_10': recall_at, 'sweep': sweep,
+            'ef': ef, 'k': k, 'recall_at_k': recall_at, 'sweep': sweep,
             'stage': 'routing_cuda + traverse_cuda (GPU search stage)',
         },
         'roofline': {
@@ -383,7 +388,7 @@ def context_figures(line, args, cfg, index, stage, query, target, ef,
     line['config']['end_to_end'] = {
         'api': 'IndexStaged.search', 'chunk_size': chunk,
         'queries_per_s': round(B / t_e2e, 1),
-        'recall_at_10': round(_utils.recall(top_I, target), 4)}
+        'recall_at_k': round(_utils.recall(top_I, target), 4)}
 
 
 if __name__ == '__main__':
