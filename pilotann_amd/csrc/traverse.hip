@@ -9,8 +9,8 @@
 //     whole wavefront advances it in lock step (uniform control flow, walks
 //     unrolled by level, scalar integer compares);
 //   * the result list is the exact set of the H best distances seen so far —
-//     what the reference's result heap holds — spread over registers,
-//     ceil(H/64) entries per lane;
+//     what the reference's result heap holds — as a flat LDS array of which
+//     the registers track the maximum and where it sits;
 //   * the visited set is exact: one bit per storage row in a per-wavefront
 //     slice of a pooled HBM bitmask (atomic OR), behind a small LDS table of
 //     rows already known to be marked;
@@ -54,9 +54,9 @@ constexpr int kSeenCache = 1 << kSeenCacheLog2;  // LDS words remembering visite
 // in lane j), bank B level 6 (lane j - 64), banks C and D the left and right
 // children of level 7 (lane (j - 128) / 2), so a sibling pair is always two
 // v_readlane of known registers.  Deeper nodes sit in LDS at [j - 256] as
-// (key, value), a sibling pair per aligned 16 bytes.  Keys are kept as order-preserving
-// integers (float_to_key) so that every comparison of a walk is a scalar
-// integer compare.  All lanes run the same, uniform, control flow; the walks
+// (key, value), a sibling pair per aligned 16 bytes.  Keys are kept as
+// order-preserving integers (float_to_key) so that every comparison of a walk
+// is a scalar integer compare.  All lanes run the same, uniform, control flow; the walks
 // are unrolled by level so that each level is a dozen instructions.  After
 // each operation the heap is, cell for cell, the reference's.  Every lane
 // stores the same values to the same LDS cells and reads the same cells, so a
