@@ -404,8 +404,10 @@ template <int S>
 struct Results {
     static constexpr int kInf = 0x7f800000;      // float_to_key(+inf)
     static constexpr int kNegInf = (int)0x807fffff;  // float_to_key(-inf)
-    int *rk;      // float_to_key of the distance, kWave * S cells
-    int *rv;
+    int *rk;      // LDS: float_to_key of the distance, kWave * S cells
+    int *rv;      // device memory: the values, same cells (written once per
+                  // insert, read at the end; every lane stores the same value
+                  // to a cell and so reads back its own store)
     int lane_max;
     int worst;    // uniform
     int pos;      // uniform: a cell whose key is `worst`
@@ -490,7 +492,7 @@ struct TraverseArgs {
     int *work_counter;
     unsigned long long *counters;
     int batch, n_nodes, n_storage, dp, n_init, k, H, deg, max_iter;
-    int words_per_slot, sort_n, lds_cells;
+    int words_per_slot, slot_stride, sort_n, lds_cells;
 };
 
 __global__ void reset_work_counter(int *counter) { *counter = 0; }
@@ -541,8 +543,8 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
         float cand_key[kWave];
         float query[DP8 ? query_floats(8 * DP8) : 4];
         int2 heap[kHeapCells];  // open list tail; the final sort reuses it
-        int res_key[S * kWave];  // result list
-        int res_val[S * kWave];
+        int res_key[S * kWave];  // result list: keys (the values are in the slot's
+                                 // memory behind the visited slice)
     };
     __shared__ __align__(16) Lds lds;
     extern __shared__ __align__(16) float query_any_length[];  // DP8 == 0 only
@@ -558,7 +560,7 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
     uint32_t *seen_cache = lds.seen_cache;
     const bool use_cache = a.n_storage <= (0xffff << kSeenCacheLog2);
     const int deg = a.deg;
-    uint32_t *seen = a.seen + (size_t)blockIdx.x * (size_t)a.words_per_slot;
+    uint32_t *seen = a.seen + (size_t)blockIdx.x * (size_t)a.slot_stride;
 
     for (;;) {
         int q = 0;
@@ -580,7 +582,8 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
         for (int i = lane; i < kSeenCache; i += kWave) seen_cache[i] = 0xffffffffu;
         open.reset(lane);
         Results<S> res;
-        res.rk = lds.res_key, res.rv = lds.res_val;
+        res.rk = lds.res_key;
+        res.rv = reinterpret_cast<int *>(seen + a.words_per_slot);
         res.init(H, lane);
         // The clearing stores must have reached the cache level where the
         // atomic ORs are performed before the first OR is issued.  Only this
@@ -908,7 +911,7 @@ TraverseFn pick_kernel(int H, int dp) {
 }
 
 struct Plan {
-    int H, sort_n, lds_cells, lds_bytes, n_slots, words_per_slot;
+    int H, sort_n, lds_cells, lds_bytes, n_slots, words_per_slot, slot_stride;
     size_t workspace_bytes;
     TraverseFn fn;
 };
@@ -967,8 +970,10 @@ int make_plan(int64_t n_storage, int64_t batch, int dp, int ef_total, Plan *p) {
     if (slots < 1) slots = 1;
     p->n_slots = (int)slots;
     p->words_per_slot = round_up((n_storage + 31) / 32, kSlotAlignWords);
+    // a slot: the visited slice, then the values of the result list
+    p->slot_stride = p->words_per_slot + round_up(p->H, kWave);
     p->workspace_bytes =
-        kWorkCounterBytes + (size_t)p->n_slots * p->words_per_slot * 4;
+        kWorkCounterBytes + (size_t)p->n_slots * p->slot_stride * 4;
     return PA_OK;
 }
 
@@ -1080,6 +1085,7 @@ extern "C" int pa_traverse(int64_t *out_I, float *out_D, const int32_t *adj,
     // traverse_cpu.cpp:18,82
     a.max_iter = 2 * beam * ef < 1024 ? 2 * beam * ef : 1024;
     a.words_per_slot = p.words_per_slot, a.sort_n = p.sort_n;
+    a.slot_stride = p.slot_stride;
     a.lds_cells = p.lds_cells;
 
     hipStream_t stream = (hipStream_t)stream_;
