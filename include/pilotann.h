@@ -198,6 +198,45 @@ int pa_pipeline(int64_t *topk_I, float *topk_D, const int64_t *full_indptr,
                 int n_neighbors, int ef_search, int k, int chunk_size,
                 void *caller_stream);
 
+/* ---- refine on the device ---------------------------------------------------- */
+
+/*
+ * `traverse_refine` (extension/traverse_cpu.cpp:261-369) run on the device
+ * instead of the host: same arguments, same two searches per query, same
+ * results (distances bit for bit, ids up to exact distance ties), with every
+ * pointer in device memory.  The reference has no device version of this
+ * stage; it is for indexes whose full-dimension rows fit device memory.
+ *
+ *   sub_adj, sub_gid, sub_mapping: the subgraph as pa_graph_prepare made it
+ *         for pa_traverse (rows of sampled-node ranks, rank -> node, node ->
+ *         rank), sub_neighbors its row length.
+ *   full_adj: the full graph from pa_graph_prepare with the identity mapping
+ *         (n_storage == n_nodes), full_neighbors its row length.
+ *   storage [n_nodes * d_model], query [batch * d_model]: full dimension.
+ *   init_I / init_D [batch * n_init]: the candidates; init_D is completed in
+ *         place.  buf_* [batch * n_buffers] receives the first search's
+ *         result and may be the same memory as init_*.  out_* [batch * k].
+ *         Where a row is longer than pa_heap_size(ef_search) the surplus
+ *         slots come first and hold -1 / -inf (traverse_cpu.cpp:150-162).
+ *   counters: NULL, or 6 uint64 device words incremented by {expansions on
+ *         the subgraph, expansions on the full graph, full-dimension
+ *         distances, candidates admitted, distances completed, adjacency
+ *         entries read}.
+ *   workspace: at least pa_refine_plan()'s bytes, 256-byte aligned, not
+ *         shared with a call that may run at the same time.
+ * Asynchronous on `stream`.
+ */
+int pa_refine_plan(int64_t n_nodes, int64_t batch, int d_model, int ef_search,
+                   int *n_slots, size_t *workspace_bytes);
+int pa_refine(int64_t *out_I, float *out_D, int64_t *buf_I, float *buf_D,
+              const int64_t *init_I, float *init_D, const int32_t *sub_adj,
+              const int32_t *sub_gid, const int64_t *sub_mapping,
+              const int32_t *full_adj, const float *storage,
+              const float *query, int64_t batch, int64_t n_nodes, int d_model,
+              int d_principle, int n_init, int n_buffers, int k, int ef_search,
+              int sub_neighbors, int full_neighbors, void *workspace,
+              size_t workspace_bytes, uint64_t *counters, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

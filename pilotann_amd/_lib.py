@@ -31,6 +31,10 @@ _SIGNATURES = {
     'pa_traverse_refine': (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                                   _vp, _vp, _vp, _vp, _i64, _i64, _int, _int,
                                   _int, _int, _int, _int]),
+    'pa_refine_plan': (_int, [_i64, _i64, _int, _int,
+                              ctypes.POINTER(_int), ctypes.POINTER(_sz)]),
+    'pa_refine': (_int, [_vp] * 12 + [_i64, _i64] + [_int] * 8 +
+                  [_vp, _sz, _vp, _vp]),
     'pa_pipeline': (_int, [_vp] * 15 + [_i64, _i64, _i64] + [_int] * 7 + [_vp]),
 }
 

@@ -89,7 +89,8 @@ __device__ __forceinline__ int wave_max_key(int x) {
 // share a row: lane a of the quad owns accumulators 2a and 2a + 1 and streams
 // its 8 bytes of every 32-byte group, so all loads of a row are in flight at
 // once in 2 * dp / 8 registers.  `row` points at the lane's pair of the first
-// group, `qv` at the lane's run of the query in LDS (query_slot layout).  Lane 0 of the quad returns the distance; every
+// group, `qv` at the lane's run of the query in LDS (query_slot layout).  Lane 0
+// of the quad returns the distance; every
 // lane of the wavefront must call this (the exchange inside the quad is a DPP
 // move), lanes without a row pass active = false.
 constexpr int kLanesPerRow = 4;
@@ -103,6 +104,26 @@ __host__ __device__ constexpr int query_run(int groups) { return groups + 2; }
 __host__ __device__ constexpr int query_floats(int dp) { return 8 * query_run(dp >> 3); }
 __device__ __forceinline__ int query_slot(int i, int groups) {
     return 2 * (((i >> 1) & 3) * query_run(groups) + (i >> 3)) + (i & 1);
+}
+
+// The eight accumulators of a row, added left to right (distance.h:50-54):
+// lane a of the quad holds accumulators 2a and 2a + 1; lane 0 of the quad
+// returns the sum.  One v_add_f32_dpp per term (the other lanes' accumulators come in as
+// the swizzled operand); the s_nop covers the two wait states a DPP read needs
+// after the last FMA wrote a0 / a1.
+__device__ __forceinline__ float quad_reduce(float a0, float a1) {
+    float s;
+    asm("s_nop 1\n\t"
+        "v_add_f32 %0, %1, %2\n\t"
+        "v_add_f32_dpp %0, %1, %0 quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf\n\t"
+        "v_add_f32_dpp %0, %2, %0 quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf\n\t"
+        "v_add_f32_dpp %0, %1, %0 quad_perm:[2,2,2,2] row_mask:0xf bank_mask:0xf\n\t"
+        "v_add_f32_dpp %0, %2, %0 quad_perm:[2,2,2,2] row_mask:0xf bank_mask:0xf\n\t"
+        "v_add_f32_dpp %0, %1, %0 quad_perm:[3,3,3,3] row_mask:0xf bank_mask:0xf\n\t"
+        "v_add_f32_dpp %0, %2, %0 quad_perm:[3,3,3,3] row_mask:0xf bank_mask:0xf"
+        : "=&v"(s)
+        : "v"(a0), "v"(a1));
+    return s;
 }
 
 template <int DP8>
@@ -145,22 +166,51 @@ __device__ __forceinline__ float quad_square_dist(const float2 *row,
             }
         }
     }
-    // accumulators 0..7 left to right: lane 0 has (0, 1), lane 1 (2, 3), ...
-    // One v_add_f32_dpp per term (the other lanes' accumulators come in as the
-    // swizzled operand); the s_nop covers the two wait states a DPP read needs
-    // after the last FMA wrote a0 / a1.
-    float s;
-    asm("s_nop 1\n\t"
-        "v_add_f32 %0, %1, %2\n\t"
-        "v_add_f32_dpp %0, %1, %0 quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf\n\t"
-        "v_add_f32_dpp %0, %2, %0 quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf\n\t"
-        "v_add_f32_dpp %0, %1, %0 quad_perm:[2,2,2,2] row_mask:0xf bank_mask:0xf\n\t"
-        "v_add_f32_dpp %0, %2, %0 quad_perm:[2,2,2,2] row_mask:0xf bank_mask:0xf\n\t"
-        "v_add_f32_dpp %0, %1, %0 quad_perm:[3,3,3,3] row_mask:0xf bank_mask:0xf\n\t"
-        "v_add_f32_dpp %0, %2, %0 quad_perm:[3,3,3,3] row_mask:0xf bank_mask:0xf"
-        : "=&v"(s)
-        : "v"(a0), "v"(a1));
-    return s;
+    return quad_reduce(a0, a1);
+}
+
+// The same sum for rows of any length (`groups` groups of eight from where
+// `row` and `qv` point): the loads of sixteen groups are in flight at once,
+// the FMAs of a group follow those of the group before it, as on the host.
+// `wide`: the lane's run in LDS is 16-byte aligned (an even number of groups
+// before it), so the query is read two groups at a time.
+__device__ __forceinline__ float quad_square_dist_long(const float2 *row,
+                                                       const float2 *qv,
+                                                       int groups, bool wide,
+                                                       bool active) {
+    float a0 = 0.f, a1 = 0.f;
+    if (active) {
+        int t = 0;
+        if (wide) {
+            constexpr int kChunk = 16;
+            for (; t + kChunk <= groups; t += kChunk) {
+                float2 x[kChunk];
+#pragma unroll
+                for (int u = 0; u < kChunk; ++u) x[u] = row[4 * (t + u)];
+                __builtin_amdgcn_sched_barrier(0);
+                const float4 *q4 = reinterpret_cast<const float4 *>(qv + t);
+#pragma unroll
+                for (int u = 0; u < kChunk; u += 2) {
+                    const float4 y = q4[u >> 1];
+                    const float d0 = y.x - x[u].x, d1 = y.y - x[u].y;
+                    a0 = fmaf(d0, d0, a0);
+                    a1 = fmaf(d1, d1, a1);
+                    const float d2 = y.z - x[u + 1].x, d3 = y.w - x[u + 1].y;
+                    a0 = fmaf(d2, d2, a0);
+                    a1 = fmaf(d3, d3, a1);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        for (; t < groups; ++t) {
+            const float2 x = row[4 * t];
+            const float2 y = qv[t];
+            const float d0 = y.x - x.x, d1 = y.y - x.y;
+            a0 = fmaf(d0, d0, a0);
+            a1 = fmaf(d1, d1, a1);
+        }
+    }
+    return quad_reduce(a0, a1);
 }
 
 }  // namespace pa

@@ -31,450 +31,11 @@
 
 #include "device_common.h"
 #include "pilotann.h"
+#include "search_lists.h"
 
 using namespace pa;
 
 namespace {
-
-constexpr int kSlotAlignWords = 256;   // bitmask slice: multiple of 1 KiB
-constexpr int kWorkCounterBytes = 256; // head of the workspace
-#ifndef PA_SEEN_LOG2
-#define PA_SEEN_LOG2 10
-#endif
-constexpr int kSeenCacheLog2 = PA_SEEN_LOG2;
-constexpr int kSeenCache = 1 << kSeenCacheLog2;  // LDS words remembering visited rows
-
-// ---- open list: heapq.cuh, top of the heap in registers ----------------------
-//
-// The reference's open list is an array heap of 2H cells with the sift rules
-// of extension/inc/heapq.cuh:13-88.  Here node i of that array is node
-// j = i + 1 (children 2j and 2j + 1), level L holds j in [2^L, 2^(L+1)).
-//
-// Levels 0..7 live in registers, one node per lane: bank A levels 0..5 (node j
-// in lane j), bank B level 6 (lane j - 64), banks C and D the left and right
-// children of level 7 (lane (j - 128) / 2), so a sibling pair is always two
-// v_readlane of known registers.  Deeper nodes sit in LDS at [j - 256] as
-// (key, value), a sibling pair per aligned 16 bytes.  Keys are kept as
-// order-preserving integers (float_to_key) so that every comparison of a walk
-// is a scalar integer compare.  All lanes run the same, uniform, control flow; the walks
-// are unrolled by level so that each level is a dozen instructions.  After
-// each operation the heap is, cell for cell, the reference's.  Every lane
-// stores the same values to the same LDS cells and reads the same cells, so a
-// lane only ever reads back its own stores and the walks need no fences.
-__device__ __forceinline__ int float_to_key(float x) {
-    const int b = __float_as_int(x);
-    return b ^ ((b >> 31) & 0x7fffffff);
-}
-__device__ __forceinline__ float key_to_float(int k) {
-    return __int_as_float(k ^ ((k >> 31) & 0x7fffffff));
-}
-
-// c + (a != b) on the scalar unit (the compiler routes the boolean of a
-// uniform compare through a vector register otherwise).
-__device__ __forceinline__ int add_if_ne(int c, int a, int b) {
-    int r;
-    asm("s_cmp_lg_u32 %1, %2\n\ts_addc_u32 %0, %3, 0"
-        : "=s"(r)
-        : "s"(a), "s"(b), "s"(c)
-        : "scc");
-    return r;
-}
-
-constexpr int floor_log2(int x) { return x <= 1 ? 0 : 1 + floor_log2(x >> 1); }
-
-// c + bit `idx` of a 64-bit lane mask, on the scalar unit.
-__device__ __forceinline__ int add_if_bit(int c, unsigned long long mask, int idx) {
-    int r;
-    asm("s_bitcmp1_b64 %1, %2\n\ts_addc_u32 %0, %3, 0"
-        : "=s"(r)
-        : "s"(mask), "s"(idx), "s"(c)
-        : "scc");
-    return r;
-}
-
-template <int H>
-struct OpenList {
-    static constexpr int kSize = 2 * H;           // cells of the reference heap
-    static constexpr int kDepth = floor_log2(kSize);  // deepest level
-    static constexpr int kRegNodes = 256;
-    static constexpr int kLdsCells = kSize + 2 > kRegNodes ? kSize + 2 - kRegNodes : 0;
-    static constexpr int kInf = 0x7f800000;       // float_to_key(+inf)
-    int Ak, Av, Bk, Bv, Ck, Cv, Dk, Dv;
-    int2 *cells;  // node j >= 256 at [j - 256] as (key, value); 16-byte aligned
-
-    __device__ __forceinline__ static int rl(int x, int l) {
-        return __builtin_amdgcn_readlane(x, l);
-    }
-    // storage class of a level: 0 bank A, 1 bank B, 2 banks C/D, 3 LDS
-    __device__ __forceinline__ static constexpr int kind(int level) {
-        return level <= 5 ? 0 : level == 6 ? 1 : level == 7 ? 2 : 3;
-    }
-
-    __device__ __forceinline__ void reset(int lane) {
-        Ak = Bk = Ck = Dk = kInf;
-        Av = Bv = Cv = Dv = -1;
-        for (int i = lane; i < kLdsCells; i += kWave) cells[i] = make_int2(kInf, -1);
-    }
-
-    // keys (and values) of the sibling pair (c, c + 1), c even, of a level.
-    // KIND and VALS are constants once the level loops are unrolled.
-    __device__ __forceinline__ void pair(const int KIND, const bool VALS, int c,
-                                         int &ka, int &kb, int &va,
-                                         int &vb) const {
-        if (KIND == 0) {
-            ka = rl(Ak, c), kb = rl(Ak, c + 1);
-            if (VALS) va = rl(Av, c), vb = rl(Av, c + 1);
-        } else if (KIND == 1) {
-            const int l = c - 64;
-            ka = rl(Bk, l), kb = rl(Bk, l + 1);
-            if (VALS) va = rl(Bv, l), vb = rl(Bv, l + 1);
-        } else if (KIND == 2) {
-            const int l = (c - 128) >> 1;
-            ka = rl(Ck, l), kb = rl(Dk, l);
-            if (VALS) va = rl(Cv, l), vb = rl(Dv, l);
-        } else {
-            // one 16-byte read: both children with their values
-            const int4 p = *reinterpret_cast<const int4 *>(cells + (c - kRegNodes));
-            if (VALS) va = uni(p.y), vb = uni(p.w);
-            ka = uni(p.x), kb = uni(p.z);
-        }
-    }
-    __device__ __forceinline__ int key_of(const int KIND, int j) const {
-        if (KIND == 0) return rl(Ak, j);
-        if (KIND == 1) return rl(Bk, j - 64);
-        if (KIND == 2) {
-            // both banks are read and one result is kept: two instructions
-            // more than a branch on the parity of j would need, no branch
-            const int l = (j - 128) >> 1;
-            const int left = rl(Ck, l), right = rl(Dk, l);
-            return (j & 1) ? right : left;
-        }
-        return uni(cells[j - kRegNodes].x);
-    }
-    __device__ __forceinline__ int val_of(const int KIND, int j) const {
-        if (KIND == 0) return rl(Av, j);
-        if (KIND == 1) return rl(Bv, j - 64);
-        if (KIND == 2) {
-            const int l = (j - 128) >> 1;
-            const int left = rl(Cv, l), right = rl(Dv, l);
-            return (j & 1) ? right : left;
-        }
-        return uni(cells[j - kRegNodes].y);
-    }
-    // lane l of a key bank and of its value bank := two uniform values
-    // (v_writelane takes one scalar register besides M0, which holds the lane)
-    __device__ __forceinline__ static void set_lane(int &kbank, int &vbank, int k,
-                                                    int v, int l) {
-        asm("s_mov_b32 m0, %4\n\t"
-            "s_nop 0\n\t"
-            "v_writelane_b32 %0, %2, m0\n\t"
-            "v_writelane_b32 %1, %3, m0"
-            : "+v"(kbank), "+v"(vbank)
-            : "s"(k), "s"(v), "s"(l)
-            : "m0");
-    }
-    __device__ __forceinline__ void put(const int KIND, int j, int k, int v,
-                                        int lane) {
-        if (KIND == 0) {
-            set_lane(Ak, Av, k, v, j);
-        } else if (KIND == 1) {
-            set_lane(Bk, Bv, k, v, j - 64);
-        } else if (KIND == 2) {
-            // lane-masked selects on both banks instead of a branch on the
-            // parity of j around two v_writelane
-            const int l = (j - 128) >> 1;
-            const bool here = lane == l;
-            const bool right = j & 1;
-            Ck = (here && !right) ? k : Ck;
-            Cv = (here && !right) ? v : Cv;
-            Dk = (here && right) ? k : Dk;
-            Dv = (here && right) ? v : Dv;
-        } else {
-            // every lane stores the same pair to the same cell: one LDS
-            // write, and no divergent branch around it
-            cells[j - kRegNodes] = make_int2(k, v);
-        }
-    }
-
-    // Which child a walk takes, for every sibling pair of the register levels
-    // at once: lane-parallel compares against the sibling (one DPP move per
-    // bank), read back as lane masks, so that a level of the walk is three
-    // scalar instructions and no register read.  LARGER selects the rule of
-    // heap_replace (strictly larger right child), else that of the sift of a
-    // pop (strictly smaller right child); left wins ties in both.  In banks A
-    // and B bit i of the mask tells about the pair whose right child sits in
-    // lane i; in banks C/D lane i holds both children.
-    struct Choice {
-        unsigned long long a, b, cd;
-    };
-    template <bool LARGER>
-    __device__ __forceinline__ Choice choices() const {
-        Choice ch;
-        const int sa = __builtin_amdgcn_update_dpp(Ak, Ak, 0xB1, 0xF, 0xF, false);
-        ch.a = __ballot(LARGER ? Ak > sa : Ak < sa);
-        ch.b = 0, ch.cd = 0;
-        if (kDepth >= 6) {
-            const int sb = __builtin_amdgcn_update_dpp(Bk, Bk, 0xB1, 0xF, 0xF, false);
-            ch.b = __ballot(LARGER ? Bk > sb : Bk < sb);
-        }
-        if (kDepth >= 7) ch.cd = __ballot(LARGER ? Dk > Ck : Dk < Ck);
-        return ch;
-    }
-    // the child of j the walk takes on register level L (1..7), L < kDepth
-    // or the pair is known to be complete: 2j + (bit of the pair in the
-    // level's mask), three scalar instructions.  s_bitcmp1_b64 looks at the
-    // low six bits of its index only, so node numbers serve as lane numbers
-    // (bank B holds node j in lane j - 64, banks C/D the children of node j
-    // in lane j - 64).
-    __device__ __forceinline__ int step_down(const int L, int j,
-                                             const Choice &ch) const {
-        int r;
-        if (kind(L) <= 1) {
-            // t = 2j + 1, the right child, whose lane holds the pair's bit
-            asm("s_lshl1_add_u32 %0, %1, 1\n\t"
-                "s_bitcmp1_b64 %2, %0\n\t"
-                "s_addc_u32 %0, %0, -1"
-                : "=&s"(r)
-                : "s"(j), "s"(kind(L) == 0 ? ch.a : ch.b)
-                : "scc");
-        } else {
-            asm("s_lshl_b32 %0, %1, 1\n\t"
-                "s_bitcmp1_b64 %2, %1\n\t"
-                "s_addc_u32 %0, %0, 0"
-                : "=&s"(r)
-                : "s"(j), "s"(ch.cd)
-                : "scc");
-        }
-        return r;
-    }
-
-    // heapq.cuh:37-45 with the sift of :13-29: the root leaves, (inf, -1)
-    // sinks along the smaller child (left on ties).  The reference stops when
-    // that child is (inf, -1) too; going on to the bottom instead only copies
-    // (inf, -1) over (inf, -1) — every infinite cell carries -1 — so the
-    // final state is the same and the walk is straight-line code.  Levels
-    // 1..kDepth-1 are complete; on level kDepth only nodes up to kSize exist
-    // and node kSize has no sibling (its absent sibling's cell holds +inf and
-    // is never the smaller one).
-    __device__ __forceinline__ void pop(int lane, int &out_k, int &out_v) {
-        out_k = rl(Ak, 1);
-        out_v = rl(Av, 1);
-        const Choice ch = choices<false>();
-        // Register levels in three passes, so that no read waits for a write
-        // of the same bank: the path (masks only), then every entry on it,
-        // then the stores.  Reading first is the same thing: a level's store
-        // goes to the cell above the one read.
-        constexpr int kRegLevels = kDepth < 7 ? kDepth : 7;
-        int node[kRegLevels + 1];
-        node[0] = 1;
-        bool cut = false;  // level kDepth has no node below node[kDepth - 1]
-#pragma unroll
-        for (int L = 1; L <= kRegLevels; ++L) {
-            if (L == kDepth && 2 * node[L - 1] > kSize) {
-                cut = true;
-                node[L] = node[L - 1];
-            } else {
-                node[L] = step_down(L, node[L - 1], ch);
-            }
-        }
-        int ck[kRegLevels + 1], cv[kRegLevels + 1];
-#pragma unroll
-        for (int L = 1; L <= kRegLevels; ++L) {
-            ck[L] = key_of(kind(L), node[L]);
-            cv[L] = val_of(kind(L), node[L]);
-        }
-#pragma unroll
-        for (int L = 1; L <= kRegLevels; ++L) {
-            if (L == kDepth && cut) {
-                put(kind(L - 1), node[L - 1], kInf, -1, lane);
-                return;
-            }
-            put(kind(L - 1), node[L - 1], ck[L], cv[L], lane);
-        }
-        int j = node[kRegLevels];
-#pragma unroll
-        for (int L = kRegLevels + 1; L <= kDepth; ++L) {
-            if (L == kDepth && 2 * j > kSize) {
-                put(kind(L - 1), j, kInf, -1, lane);
-                return;
-            }
-            int ka, kb, va, vb;
-            pair(3, true, 2 * j, ka, kb, va, vb);
-            if (L == kDepth) kb = 2 * j == kSize ? ka : kb;
-            const int k = min(ka, kb);
-            const int v = k != ka ? vb : va;
-            const int c = add_if_ne(2 * j, k, ka);
-            put(kind(L - 1), j, k, v, lane);
-            j = c;
-        }
-        put(kind(kDepth), j, kInf, -1, lane);
-    }
-
-    // heapq.cuh:47-77: walk to a leaf through the larger child (left on
-    // ties), overwrite it when the new key is strictly smaller, let the new
-    // entry rise.  In two parts so that the caller can put independent work
-    // between them: the walk is straight-line code, the rise branches.
-    struct Leaf {
-        int j;       // the leaf
-        int key;     // its key
-        bool bottom; // it is on level kDepth
-    };
-    __device__ __forceinline__ Leaf walk_to_large_leaf() const {
-        const Choice ch = choices<true>();
-        int j = 1;
-        bool bottom = true;  // the walk reached level kDepth
-        int walked_key = 0;  // key of node j when its level is an LDS level
-#pragma unroll
-        for (int L = 1; L <= kDepth; ++L) {
-            if (L == kDepth && 2 * j > kSize) {
-                bottom = false;
-                break;
-            }
-            if (kind(L) <= 2) {
-                // node kSize has no sibling: the left child it is
-                j = (L == kDepth && 2 * j == kSize) ? 2 * j : step_down(L, j, ch);
-            } else {
-                int ka, kb, va, vb;
-                pair(3, false, 2 * j, ka, kb, va, vb);
-                if (L == kDepth) kb = 2 * j == kSize ? ka : kb;
-                walked_key = max(ka, kb);
-                j = add_if_ne(2 * j, walked_key, ka);
-            }
-        }
-        // the leaf's key: the walk has it already when the leaf is in LDS
-        Leaf leaf;
-        leaf.j = j, leaf.bottom = bottom;
-        if (bottom)
-            leaf.key = kind(kDepth) == 3 ? walked_key : key_of(kind(kDepth), j);
-        else
-            leaf.key = kind(kDepth - 1) == 3 ? walked_key : key_of(kind(kDepth - 1), j);
-        return leaf;
-    }
-    // SPARSE: the heap is nearly empty (the entries of a query are pushed),
-    // so most ancestors of the leaf are (inf, -1), and so is everything below
-    // such an ancestor: moving it down would write (inf, -1) over (inf, -1)
-    // and is left out.
-    template <bool SPARSE = false>
-    __device__ __forceinline__ void replace_leaf(const Leaf &leaf, int k, int v,
-                                                 int lane) {
-        if (k >= leaf.key) return;
-        int j = leaf.j;
-        // one store per level: the parent's entry while it is larger than
-        // the new key, the new entry where the rise stops
-        auto rise = [&](const int L) -> bool {
-            const int up = j >> 1;
-            const int pk = key_of(kind(L - 1), up);
-            if (SPARSE && pk == kInf) {
-                j = up;
-                return false;
-            }
-            const int pv = val_of(kind(L - 1), up);
-            const bool stop = pk <= k;
-            put(kind(L), j, stop ? k : pk, stop ? v : pv, lane);
-            j = up;
-            return stop;
-        };
-        if (leaf.bottom && rise(kDepth)) return;
-#pragma unroll
-        for (int L = kDepth - 1; L >= 1; --L)
-            if (rise(L)) return;
-        put(0, 1, k, v, lane);
-    }
-    template <bool SPARSE = false>
-    __device__ __forceinline__ void replace(int k, int v, int lane) {
-        const Leaf leaf = walk_to_large_leaf();
-        replace_leaf<SPARSE>(leaf, k, v, lane);
-    }
-};
-
-// ---- result list: the H smallest distances ------------------------------------
-//
-// The reference keeps them in a heap of negated keys whose root is the worst
-// kept (traverse_cpu.cpp:21-39): a candidate enters iff its distance is
-// strictly below that root, and replaces it.  Which array cell holds what has
-// no effect on the search; only the set and its maximum do.  Here the cells
-// are a flat LDS array, S per lane (lane l owns cells l*S .. l*S+S-1), of which
-// the registers keep only each lane's maximum, the wavefront's maximum and the
-// position of one cell that holds it: an insert is one store to that cell,
-// one read of every lane's own cells and a wavefront maximum.  Empty cells
-// hold +inf (so the maximum is +inf until H candidates came), cells beyond H
-// hold -inf and never win.
-
-template <int S>
-struct Results {
-    static constexpr int kInf = 0x7f800000;      // float_to_key(+inf)
-    static constexpr int kNegInf = (int)0x807fffff;  // float_to_key(-inf)
-    int *rk;      // LDS: float_to_key of the distance, kWave * S cells
-    int *rv;      // device memory: the values, same cells (written once per
-                  // insert, read at the end; every lane stores the same value
-                  // to a cell and so reads back its own store)
-    int lane_max;
-    int worst;    // uniform
-    int pos;      // uniform: a cell whose key is `worst`
-
-    __device__ __forceinline__ void init(int H, int lane) {
-        lane_max = kNegInf;
-#pragma unroll
-        for (int s = 0; s < S; ++s) {
-            const int c = lane * S + s;
-            const int k = c < H ? kInf : kNegInf;
-            rk[c] = k, rv[c] = -1;
-            lane_max = max(lane_max, k);
-        }
-        worst = kInf;
-        pos = 0;
-    }
-    // Caller has checked k < worst.  In two parts so that the caller can put
-    // independent work between the LDS traffic and its use.
-    __device__ __forceinline__ void begin_insert(int k, int v, int lane, int (&key)[S]) {
-        // Every lane stores the same pair to the same cell, so the lane that
-        // owns the cell reads back its own store: program order is enough.
-        rk[pos] = k, rv[pos] = v;
-#pragma unroll
-        for (int s = 0; s < S; ++s) key[s] = rk[lane * S + s];
-    }
-    __device__ __forceinline__ void finish_insert(int lane, const int (&key)[S]) {
-        int m = key[0];
-#pragma unroll
-        for (int s = 1; s < S; ++s) m = max(m, key[s]);
-        lane_max = m;
-        worst = wave_max_key(lane_max);
-        // the first lane that holds the new maximum, its first such cell
-        const int holder = __builtin_ctzll(__ballot(lane_max == worst));
-        int c = lane * S + S - 1;
-#pragma unroll
-        for (int s = S - 2; s >= 0; --s) c = key[s] == worst ? lane * S + s : c;
-        pos = __builtin_amdgcn_readlane(c, holder);
-    }
-    __device__ __forceinline__ void insert(int k, int v, int lane) {
-        int key[S];
-        begin_insert(k, v, lane, key);
-        finish_insert(lane, key);
-    }
-};
-
-// ---- distances ---------------------------------------------------------------
-
-// Squared L2 from the query (LDS) to the storage rows listed in cand_id[0..n),
-// written to cand_key: 16 rows per pass, four lanes per row.
-template <int DP8>
-__device__ __forceinline__ void eval_rows(const float *__restrict__ storage,
-                                          const float *qv, const int *cand_id,
-                                          float *cand_key, int n, int dp,
-                                          int lane) {
-    const int quad = lane >> 2, part = lane & 3;
-    const float2 *qq = reinterpret_cast<const float2 *>(qv) + part * query_run(dp >> 3);
-    for (int base = 0; base < n; base += kRowsPerPass) {
-        const int c = base + quad;
-        const bool active = c < n;
-        const float2 *row = reinterpret_cast<const float2 *>(storage);
-        if (active)
-            row = reinterpret_cast<const float2 *>(
-                      storage + (size_t)cand_id[c] * (size_t)dp) + part;
-        const float s = quad_square_dist<DP8>(row, qq, dp >> 3, active);
-        if (active && part == 0) cand_key[c] = s;
-    }
-}
 
 // ---- the search ---------------------------------------------------------------
 

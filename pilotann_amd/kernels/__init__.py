@@ -345,6 +345,94 @@ def traverse_refine(output_I: torch.Tensor,
         output_I.size(-1), int(ef_search)), 'pa_traverse_refine')
 
 
+def prepare_full_graph(indptr, indices, n_neighbors=None):
+    """:class:`PreparedGraph` of a graph in which every node has a row (the
+    full graph of the refine): identity mapping.  ``n_neighbors`` defaults to
+    the longest row."""
+    _check(indptr, 'indptr', 1, torch.int64, True)
+    n_nodes = indptr.size(0) - 1
+    if n_neighbors is None:
+        n_neighbors = int((indptr[1:] - indptr[:-1]).max().item())
+    key = ('identity', str(indptr.device), n_nodes)
+    mapping = _identity_maps.get(key)
+    if mapping is None:
+        mapping = torch.arange(n_nodes, dtype=torch.int64,
+                               device=indptr.device)
+        _identity_maps[key] = mapping
+    return prepare_graph(indptr, indices, mapping, n_nodes, n_neighbors)
+
+
+_identity_maps = {}
+
+
+def traverse_refine_cuda(output_I: torch.Tensor,
+                         output_D: torch.Tensor,
+                         buffer_I: torch.Tensor,
+                         buffer_D: torch.Tensor,
+                         initial_I: torch.Tensor,
+                         initial_D: torch.Tensor,
+                         subgraph: PreparedGraph,
+                         fullgraph: PreparedGraph,
+                         storage: torch.Tensor,
+                         query: torch.Tensor,
+                         ef_search: int,
+                         d_principle: int,
+                         counters: torch.Tensor = None):
+    """:func:`traverse_refine` on the device: the arguments of
+    ``kernels.traverse_refine`` (``pilot_ann/kernels/__init__.py:78-94``) as
+    device tensors, the two graphs in their prepared form (``subgraph`` from
+    :func:`prepare_graph` as the traversal uses it, ``fullgraph`` from
+    :func:`prepare_full_graph`).  Same results as the host function;
+    ``initial_D`` is completed in place, ``buffer_*`` may be ``initial_*``.
+    Enqueued on the current stream.  ``counters``: optional 6 int64."""
+    _check(query, 'query', 2, torch.float32, True)
+    _check(storage, 'storage', 2, torch.float32, True)
+    _check(initial_I, 'initial_I', 2, torch.int64, True)
+    _check(initial_D, 'initial_D', 2, torch.float32, True)
+    _check(buffer_I, 'buffer_I', 2, torch.int64, True)
+    _check(buffer_D, 'buffer_D', 2, torch.float32, True)
+    _check(output_I, 'output_I', 2, torch.int64, True)
+    _check(output_D, 'output_D', 2, torch.float32, True)
+    batch_size, d_model = query.shape
+    n_nodes = storage.size(0)
+    _require(storage.size(-1) == d_model, 'storage.size(-1) == d_model')
+    _require(output_I.size(0) == batch_size, 'output_I.size(0) == batch_size')
+    _require(buffer_I.size(0) == batch_size, 'buffer_I.size(0) == batch_size')
+    _require(initial_I.size(0) == batch_size,
+             'initial_I.size(0) == batch_size')
+    _require(output_I.size() == output_D.size(),
+             'output_I.sizes() == output_D.sizes()')
+    _require(buffer_I.size() == buffer_D.size(),
+             'buffer_I.sizes() == buffer_D.sizes()')
+    _require(initial_I.size() == initial_D.size(),
+             'initial_I.sizes() == initial_D.sizes()')
+    _require(ef_search <= 2048, 'ef_search supported')
+    _require(d_model % 8 == 0 and d_principle % 8 == 0,
+             'd_model % 8 == 0 and d_principle % 8 == 0')
+    _require(subgraph.n_nodes == n_nodes, 'subgraph.n_nodes == n_storage')
+    _require(fullgraph.n_nodes == n_nodes == fullgraph.n_storage,
+             'fullgraph.n_nodes == n_storage')
+    if counters is not None:
+        _check(counters, 'counters', 1, torch.int64, True)
+        _require(counters.numel() >= 6, 'counters.numel() >= 6')
+    lib = _lib.lib()
+    with torch.cuda.device(query.device):
+        nbytes = ctypes.c_size_t()
+        _lib.check(lib.pa_refine_plan(
+            n_nodes, batch_size, d_model, int(ef_search), None,
+            ctypes.byref(nbytes)), 'pa_refine_plan')
+        ws = _workspace(query.device, nbytes.value)
+        _lib.check(lib.pa_refine(
+            _ptr(output_I), _ptr(output_D), _ptr(buffer_I), _ptr(buffer_D),
+            _ptr(initial_I), _ptr(initial_D), _ptr(subgraph.adj),
+            _ptr(subgraph.gid), _ptr(subgraph.mapping), _ptr(fullgraph.adj),
+            _ptr(storage), _ptr(query), batch_size, n_nodes, d_model,
+            int(d_principle), initial_I.size(-1), buffer_I.size(-1),
+            output_I.size(-1), int(ef_search), subgraph.n_neighbors,
+            fullgraph.n_neighbors, _ptr(ws), ws.numel(), _ptr(counters),
+            _stream()), 'pa_refine')
+
+
 def pipeline(graph: list,
              subgraph: list,
              subgraph_cuda: list,
