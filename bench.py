@@ -214,6 +214,10 @@ def main():
                          'fourfold batch, end-to-end search), so that a '
                          'kernel trace of the run holds the timed launches '
                          'only')
+    ap.add_argument('--device-refine-only', action='store_true',
+                    help='only measure the search with the refine on the '
+                         'device and the refine kernel alone (needs --ef), '
+                         'print those figures and exit')
     ap.add_argument('--copy-calibration', action='store_true',
                     help='only run a plain 1 GiB device copy five times (to '
                          'scale the FETCH_SIZE / WRITE_SIZE counters) and exit')
@@ -248,6 +252,13 @@ def main():
     index, query, target = build_index(cfg, device)
     stage = Stage(index, query, device)
     B, k, dp = stage.B, cfg['k'], cfg['dp']
+
+    if args.device_refine_only:
+        if not args.ef:
+            ap.error('--device-refine-only needs --ef')
+        print(json.dumps(device_refine_figures(cfg, index, stage, query,
+                                               target, args.ef)), flush=True)
+        return
 
     # pick ef: smallest of the sweep with end-to-end recall@k >= 0.90
     sweep = []
@@ -382,13 +393,88 @@ def context_figures(line, args, cfg, index, stage, query, target, ef,
     chunk = 1000 if B % 1000 == 0 else B
     index.search(query, k=k, ef_search=ef, chunk_size=chunk)
     t0 = time.perf_counter()
-    top_I, _ = index.search(query, k=k, ef_search=ef, chunk_size=chunk)
+    top_I, top_D = index.search(query, k=k, ef_search=ef, chunk_size=chunk)
     t_e2e = time.perf_counter() - t0
     from pilotann_amd import utils as _utils
     line['config']['end_to_end'] = {
         'api': 'IndexStaged.search', 'chunk_size': chunk,
         'queries_per_s': round(B / t_e2e, 1),
         'recall_at_k': round(_utils.recall(top_I, target), 4)}
+    line['config']['end_to_end_device_refine'] = device_refine_figures(
+        cfg, index, stage, query, target, ef, (top_I, top_D))
+
+
+def device_refine_figures(cfg, index, stage, query, target, ef, host_top=None):
+    """The whole search with the refine on the device as well
+    (`IndexStaged.search(..., refine='device')`: the full-dimension rows and
+    the full graph resident in HBM, one launch per stage, top-k copied back),
+    and the refine kernel alone on the traversal's candidates."""
+    from pilotann_amd import utils as _utils
+    B, k, dp, d, device = stage.B, cfg['k'], cfg['dp'], cfg['d'], stage.device
+    kernels = stage.kernels
+    index.stage_refine()
+    # same rotated query as the host path: results must agree
+    same_I, same_D = index.search(query, k=k, ef_search=ef, refine='device')
+    agree = None
+    if host_top is not None:
+        agree = {
+            'distances_identical': bool(torch.equal(same_D, host_top[1])),
+            'rows_with_identical_ids': round(float(
+                (same_I == host_top[0]).all(-1).float().mean()), 4)}
+    query_dev = query.to(device)
+    index.search(query_dev, k=k, ef_search=ef, refine='device')
+    torch.cuda.synchronize()
+    reps = 5
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        top_I, _ = index.search(query_dev, k=k, ef_search=ef, refine='device')
+    t_all = (time.perf_counter() - t0) / reps
+
+    # the refine kernel alone
+    EP_I, EP_D = stage.entries()
+    cand_I, cand_D = stage.traverse(ef, EP_I, EP_D)
+    cand_I, cand_D = cand_I.flatten(1).clone(), cand_D.flatten(1).clone()
+    sub = stage.graph
+    full = kernels.prepare_full_graph(index.fullgraph_cuda.indptr,
+                                      index.fullgraph_cuda.indices)
+    q_full = stage.query_rot.to(device).contiguous()
+    init_I, init_D = cand_I.clone(), cand_D.clone()
+    buf_I, buf_D = torch.empty_like(cand_I), torch.empty_like(cand_D)
+    out_I = torch.empty(B, k, dtype=torch.long, device=device)
+    out_D = torch.empty(B, k, dtype=torch.float, device=device)
+    counters = torch.zeros(6, dtype=torch.long, device=device)
+    times = []
+    for i in range(4):
+        init_D.copy_(cand_D)
+        a, b = (torch.cuda.Event(enable_timing=True) for _ in range(2))
+        a.record()
+        kernels.traverse_refine_cuda(
+            out_I, out_D, buf_I, buf_D, init_I, init_D, sub, full,
+            index.storage_full_cuda, q_full, ef, dp,
+            counters=counters if i == 0 else None)
+        b.record()
+        torch.cuda.synchronize()
+        times.append(a.elapsed_time(b))
+    ms = float(np.mean(times[1:]))
+    c = dict(zip(['expanded_subgraph', 'expanded_full', 'distances',
+                  'admitted', 'completed', 'adjacency_entries'],
+                 counters.cpu().tolist()))
+    n_cand = cand_I.size(1)
+    # query + candidates read + completed tails + adjacency ids + full rows
+    # (4-byte id each) + buffer and top-k written
+    nbytes = (B * 4 * d + B * n_cand * 8 + c['completed'] * 4 * (d - dp)
+              + c['adjacency_entries'] * 4 + c['distances'] * (4 + 4 * d)
+              + B * (n_cand + k) * 8)
+    return {
+        'api': "IndexStaged.search(refine='device')",
+        'queries_per_s': round(B / t_all, 1),
+        'recall_at_k': round(_utils.recall(top_I, target), 4),
+        'against_host_refine': agree,
+        'refine_kernel_ms': round(ms, 3),
+        'refine_counters': c,
+        'refine_algorithmic_bytes': int(nbytes),
+        'refine_achieved_GBps': round(nbytes / (ms * 1e-3) / 1e9, 1),
+        'refine_frac_of_hbm_peak': round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
 
 
 if __name__ == '__main__':

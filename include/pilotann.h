@@ -212,7 +212,8 @@ int pa_pipeline(int64_t *topk_I, float *topk_D, const int64_t *full_indptr,
  *         rank), sub_neighbors its row length.
  *   full_adj: the full graph from pa_graph_prepare with the identity mapping
  *         (n_storage == n_nodes), full_neighbors its row length.
- *   storage [n_nodes * d_model], query [batch * d_model]: full dimension.
+ *   storage [n_nodes * d_model]: all rows in full dimension, in the layout
+ *         of pa_rows_prepare.   query [batch * d_model] (plain).
  *   init_I / init_D [batch * n_init]: the candidates; init_D is completed in
  *         place.  buf_* [batch * n_buffers] receives the first search's
  *         result and may be the same memory as init_*.  out_* [batch * k].
@@ -225,7 +226,16 @@ int pa_pipeline(int64_t *topk_I, float *topk_D, const int64_t *full_indptr,
  *   workspace: at least pa_refine_plan()'s bytes, 256-byte aligned, not
  *         shared with a call that may run at the same time.
  * Asynchronous on `stream`.
+ *
+ * pa_rows_prepare copies plain rows src [n_rows * d_model] into dst (another
+ * buffer of the same size) in the layout the refine streams: within every 16
+ * floats (two groups of eight) the four 8-byte pairs of the first group and
+ * those of the second are interleaved, pair a of both next to each other, so
+ * that a lane reads its share of two groups with one 16-byte load.  A last
+ * group without a partner stays as it is.
  */
+int pa_rows_prepare(float *dst, const float *src, int64_t n_rows, int d_model,
+                    void *stream);
 int pa_refine_plan(int64_t n_nodes, int64_t batch, int d_model, int ef_search,
                    int *n_slots, size_t *workspace_bytes);
 int pa_refine(int64_t *out_I, float *out_D, int64_t *buf_I, float *buf_D,

@@ -31,6 +31,7 @@ _SIGNATURES = {
     'pa_traverse_refine': (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                                   _vp, _vp, _vp, _vp, _i64, _i64, _int, _int,
                                   _int, _int, _int, _int]),
+    'pa_rows_prepare': (_int, [_vp, _vp, _i64, _int, _vp]),
     'pa_refine_plan': (_int, [_i64, _i64, _int, _int,
                               ctypes.POINTER(_int), ctypes.POINTER(_sz)]),
     'pa_refine': (_int, [_vp] * 12 + [_i64, _i64] + [_int] * 8 +

@@ -169,46 +169,69 @@ __device__ __forceinline__ float quad_square_dist(const float2 *row,
     return quad_reduce(a0, a1);
 }
 
-// The same sum for rows of any length (`groups` groups of eight from where
-// `row` and `qv` point): the loads of sixteen groups are in flight at once,
-// the FMAs of a group follow those of the group before it, as on the host.
-// `wide`: the lane's run in LDS is 16-byte aligned (an even number of groups
-// before it), so the query is read two groups at a time.
-__device__ __forceinline__ float quad_square_dist_long(const float2 *row,
-                                                       const float2 *qv,
-                                                       int groups, bool wide,
-                                                       bool active) {
+// Long rows (the full-dimension refine) are kept in device memory with the
+// two groups of every 64-byte block interleaved by lane: the 16 bytes lane a
+// of a quad needs of groups 2b and 2b + 1 (its pair of each) are adjacent, at
+// floats 16b + 4a .. 16b + 4a + 3, so a lane streams a row with 16-byte loads
+// and a quad covers 64 contiguous bytes per instruction — half the memory
+// instructions of the plain layout, which is what bounds a kernel that streams
+// 3 KB rows.  A last group without a partner (d / 8 odd) stays plain.
+// Position of lane a's pair of group g in a row of `groups` groups:
+__host__ __device__ constexpr int row_pair_slot(int g, int a, int groups) {
+    return (g == groups - 1 && (groups & 1)) ? 8 * g + 2 * a
+                                             : 16 * (g >> 1) + 4 * a + 2 * (g & 1);
+}
+
+// Squared L2 over groups [first, groups) of such a row (the accumulators start
+// at zero at `first`), in the host's order as above: the FMAs of a group
+// follow those of the group before it.  `row` is the row's start, `qrun` the
+// lane's run of the query in LDS (query_slot layout), `part` the lane's place
+// in its quad.  Eight blocks (16 groups) of loads are in flight at once.
+// Lane 0 of the quad returns the sum; every lane must call this.
+#ifndef PA_LONG_CHUNK
+#define PA_LONG_CHUNK 8
+#endif
+__device__ __forceinline__ float quad_square_dist_long(const float *row,
+                                                       const float2 *qrun,
+                                                       int groups, int first,
+                                                       int part, bool active) {
     float a0 = 0.f, a1 = 0.f;
     if (active) {
-        int t = 0;
-        if (wide) {
-            constexpr int kChunk = 16;
-            for (; t + kChunk <= groups; t += kChunk) {
-                float2 x[kChunk];
+        auto one_group = [&](int g) {
+            const float2 x = *reinterpret_cast<const float2 *>(
+                row + row_pair_slot(g, part, groups));
+            const float2 y = qrun[g];
+            const float d0 = y.x - x.x, d1 = y.y - x.y;
+            a0 = fmaf(d0, d0, a0);
+            a1 = fmaf(d1, d1, a1);
+        };
+        int g = first;
+        // the query is read 16 bytes at a time: the run must start 16-byte
+        // aligned, which it does when the number of groups is even
+        if ((groups & 1) == 0) {
+            if (g & 1) one_group(g++);
+            constexpr int kChunk = PA_LONG_CHUNK;  // blocks per batch of loads
+            const float4 *r4 = reinterpret_cast<const float4 *>(row) + part;
+            const float4 *q4 = reinterpret_cast<const float4 *>(qrun);
+            for (; g + 2 * kChunk <= groups; g += 2 * kChunk) {
+                float4 x[kChunk];
 #pragma unroll
-                for (int u = 0; u < kChunk; ++u) x[u] = row[4 * (t + u)];
+                for (int u = 0; u < kChunk; ++u) x[u] = r4[4 * ((g >> 1) + u)];
                 __builtin_amdgcn_sched_barrier(0);
-                const float4 *q4 = reinterpret_cast<const float4 *>(qv + t);
 #pragma unroll
-                for (int u = 0; u < kChunk; u += 2) {
-                    const float4 y = q4[u >> 1];
+                for (int u = 0; u < kChunk; ++u) {
+                    const float4 y = q4[(g >> 1) + u];
                     const float d0 = y.x - x[u].x, d1 = y.y - x[u].y;
                     a0 = fmaf(d0, d0, a0);
                     a1 = fmaf(d1, d1, a1);
-                    const float d2 = y.z - x[u + 1].x, d3 = y.w - x[u + 1].y;
+                    const float d2 = y.z - x[u].z, d3 = y.w - x[u].w;
                     a0 = fmaf(d2, d2, a0);
                     a1 = fmaf(d3, d3, a1);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
-        for (; t < groups; ++t) {
-            const float2 x = row[4 * t];
-            const float2 y = qv[t];
-            const float d0 = y.x - x.x, d1 = y.y - x.y;
-            a0 = fmaf(d0, d0, a0);
-            a1 = fmaf(d1, d1, a1);
-        }
+        for (; g < groups; ++g) one_group(g);
     }
     return quad_reduce(a0, a1);
 }

@@ -55,25 +55,38 @@ __global__ void reset_refine_counter(int *counter) { *counter = 0; }
 // rows listed in cand_id[0..n), written to cand_key: 16 rows per pass, four
 // lanes per row; the accumulators start at zero at `from`
 // (extension/inc/distance.h:31-55 called with an offset, traverse_cpu.cpp:56-59).
+// Rows are in the interleaved layout of pa_rows_prepare.
 __device__ __forceinline__ void eval_rows_from(const float *__restrict__ storage,
                                                const float *qv, const int *cand_id,
                                                float *cand_key, int n, int d,
                                                int from, int lane) {
     const int quad = lane >> 2, part = lane & 3;
-    const int groups = d >> 3, first = from >> 3;
-    const bool wide = ((groups | first) & 1) == 0;
-    const float2 *qq =
-        reinterpret_cast<const float2 *>(qv) + part * query_run(groups) + first;
+    const int groups = d >> 3;
+    const float2 *qrun =
+        reinterpret_cast<const float2 *>(qv) + part * query_run(groups);
     for (int base = 0; base < n; base += kRowsPerPass) {
         const int c = base + quad;
         const bool active = c < n;
-        const float2 *row = reinterpret_cast<const float2 *>(storage);
-        if (active)
-            row = reinterpret_cast<const float2 *>(
-                      storage + (size_t)cand_id[c] * (size_t)d + from) + part;
-        const float s = quad_square_dist_long(row, qq, groups - first, wide, active);
+        const float *row = storage;
+        if (active) row = storage + (size_t)cand_id[c] * (size_t)d;
+        const float s =
+            quad_square_dist_long(row, qrun, groups, from >> 3, part, active);
         if (active && part == 0) cand_key[c] = s;
     }
+}
+
+// Plain rows -> the interleaved layout (row_pair_slot); one thread per pair.
+__global__ void interleave_rows(const float *__restrict__ src,
+                                float *__restrict__ dst, int64_t n_pairs,
+                                int groups) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n_pairs) return;
+    const int per_row = groups * 4;
+    const int64_t r = i / per_row;
+    const int p = (int)(i - r * per_row);  // pair p of the row: group p / 4, lane p % 4
+    const float2 v = reinterpret_cast<const float2 *>(src)[i];
+    *reinterpret_cast<float2 *>(dst + r * (int64_t)groups * 8 +
+                                row_pair_slot(p >> 2, p & 3, groups)) = v;
 }
 
 #define PA_REFINE_OCCUPANCY(H) \
@@ -403,6 +416,19 @@ int make_plan(int64_t n_nodes, int64_t batch, int d, int ef_search, Plan *p) {
 }
 
 }  // namespace
+
+extern "C" int pa_rows_prepare(float *dst, const float *src, int64_t n_rows,
+                               int d_model, void *stream_) {
+    if (n_rows < 0) return PA_E_SHAPE;
+    if (d_model <= 0 || d_model % 8) return PA_E_DIM;
+    if (n_rows == 0) return PA_OK;
+    if (!dst || !src || dst == src) return PA_E_NULL;
+    const int64_t n_pairs = n_rows * (d_model / 2);
+    if ((n_pairs + 255) / 256 >= (1ll << 31)) return PA_E_RANGE;
+    interleave_rows<<<(unsigned)((n_pairs + 255) / 256), 256, 0,
+                      (hipStream_t)stream_>>>(src, dst, n_pairs, d_model / 8);
+    return (int)hipGetLastError();
+}
 
 extern "C" int pa_refine_plan(int64_t n_nodes, int64_t batch, int d_model,
                               int ef_search, int *n_slots,

@@ -365,6 +365,26 @@ def prepare_full_graph(indptr, indices, n_neighbors=None):
 _identity_maps = {}
 
 
+class PreparedRows:
+    """Full-dimension rows in the layout the device refine streams (see
+    ``pa_rows_prepare``): ``rows[n, d]`` float32 on the device, the pairs of
+    every two groups of eight interleaved by lane."""
+
+    def __init__(self, storage: torch.Tensor):
+        _check(storage, 'storage', 2, torch.float32, True)
+        _require(storage.size(-1) % 8 == 0, 'd_model % 8 == 0')
+        self.n_rows, self.d_model = storage.shape
+        self.rows = torch.empty_like(storage)
+        with torch.cuda.device(storage.device):
+            _lib.check(_lib.lib().pa_rows_prepare(
+                _ptr(self.rows), _ptr(storage), self.n_rows, self.d_model,
+                _stream()), 'pa_rows_prepare')
+
+
+def prepare_rows(storage: torch.Tensor) -> PreparedRows:
+    return PreparedRows(storage)
+
+
 def traverse_refine_cuda(output_I: torch.Tensor,
                          output_D: torch.Tensor,
                          buffer_I: torch.Tensor,
@@ -373,7 +393,7 @@ def traverse_refine_cuda(output_I: torch.Tensor,
                          initial_D: torch.Tensor,
                          subgraph: PreparedGraph,
                          fullgraph: PreparedGraph,
-                         storage: torch.Tensor,
+                         storage: PreparedRows,
                          query: torch.Tensor,
                          ef_search: int,
                          d_principle: int,
@@ -382,11 +402,13 @@ def traverse_refine_cuda(output_I: torch.Tensor,
     ``kernels.traverse_refine`` (``pilot_ann/kernels/__init__.py:78-94``) as
     device tensors, the two graphs in their prepared form (``subgraph`` from
     :func:`prepare_graph` as the traversal uses it, ``fullgraph`` from
-    :func:`prepare_full_graph`).  Same results as the host function;
+    :func:`prepare_full_graph`), the rows from :func:`prepare_rows`.  Same
+    results as the host function;
     ``initial_D`` is completed in place, ``buffer_*`` may be ``initial_*``.
     Enqueued on the current stream.  ``counters``: optional 6 int64."""
     _check(query, 'query', 2, torch.float32, True)
-    _check(storage, 'storage', 2, torch.float32, True)
+    if not isinstance(storage, PreparedRows):
+        raise RuntimeError('storage must come from prepare_rows')
     _check(initial_I, 'initial_I', 2, torch.int64, True)
     _check(initial_D, 'initial_D', 2, torch.float32, True)
     _check(buffer_I, 'buffer_I', 2, torch.int64, True)
@@ -394,8 +416,8 @@ def traverse_refine_cuda(output_I: torch.Tensor,
     _check(output_I, 'output_I', 2, torch.int64, True)
     _check(output_D, 'output_D', 2, torch.float32, True)
     batch_size, d_model = query.shape
-    n_nodes = storage.size(0)
-    _require(storage.size(-1) == d_model, 'storage.size(-1) == d_model')
+    n_nodes = storage.n_rows
+    _require(storage.d_model == d_model, 'storage.size(-1) == d_model')
     _require(output_I.size(0) == batch_size, 'output_I.size(0) == batch_size')
     _require(buffer_I.size(0) == batch_size, 'buffer_I.size(0) == batch_size')
     _require(initial_I.size(0) == batch_size,
@@ -426,7 +448,7 @@ def traverse_refine_cuda(output_I: torch.Tensor,
             _ptr(output_I), _ptr(output_D), _ptr(buffer_I), _ptr(buffer_D),
             _ptr(initial_I), _ptr(initial_D), _ptr(subgraph.adj),
             _ptr(subgraph.gid), _ptr(subgraph.mapping), _ptr(fullgraph.adj),
-            _ptr(storage), _ptr(query), batch_size, n_nodes, d_model,
+            _ptr(storage.rows), _ptr(query), batch_size, n_nodes, d_model,
             int(d_principle), initial_I.size(-1), buffer_I.size(-1),
             output_I.size(-1), int(ef_search), subgraph.n_neighbors,
             fullgraph.n_neighbors, _ptr(ws), ws.numel(), _ptr(counters),

@@ -25,6 +25,9 @@ class IndexStaged(nn.Module):
     ``seed`` and ``build_device`` are additions: every random choice of the
     build is seeded, and the build-time matrix products run where
     ``build_device`` says (the search-time split is the reference's).
+    So are :meth:`stage_refine` and ``search(..., refine='device')``: with the
+    full-dimension rows and the full graph on the device as well, the refine
+    runs there too and gives the host refine's results.
     """
 
     def __init__(self, d_model: int, d_principle: int, sample_ratio: float,
@@ -52,6 +55,9 @@ class IndexStaged(nn.Module):
         self.storage_cuda = None
         self.subgraph_cuda = None
         self.mapping_cuda = None
+        self.fullgraph_cuda = None
+        self.storage_full_cuda = None
+        self.VT_cuda = None
 
     # -- checkpoint: layers/staged.py:59-122 ---------------------------------
     @classmethod
@@ -115,6 +121,21 @@ class IndexStaged(nn.Module):
                 self.mapping_cuda, self.storage_cuda.size(0), self.n_neighbors)
         return self
 
+    def stage_refine(self):
+        """Copies what the refine needs to the device chosen by :meth:`to`:
+        all rows in full dimension, the full graph (prepared once) and the
+        rotation."""
+        device = self.cuda_device
+        assert device is not None, 'call .to(device) first'
+        self.storage_full_cuda = kernels.prepare_rows(
+            self.storage.to(device).contiguous())
+        self.VT_cuda = self.VT.to(device)
+        self.fullgraph_cuda = GraphModule(self.fullgraph.indptr,
+                                          self.fullgraph.indices).to(device)
+        kernels.prepare_full_graph(self.fullgraph_cuda.indptr,
+                                   self.fullgraph_cuda.indices)
+        return self
+
     # -- build: layers/staged.py:141-189 --------------------------------------
     def train(self, x: torch.Tensor):
         assert x.dim() == 2
@@ -151,8 +172,11 @@ class IndexStaged(nn.Module):
     # -- search: layers/staged.py:191-228 -------------------------------------
     @torch.no_grad()
     def search(self, query: torch.Tensor, k: int, ef_search: int,
-               chunk_size: int = 128):
+               chunk_size: int = 128, refine: str = 'host'):
         assert query.dim() == 2
+        if refine == 'device':
+            return self._search_on_device(query, k, ef_search)
+        assert refine == 'host'
         query = torch.matmul(query, self.VT.T).contiguous()
         query_cuda = query[:, :self.d_principle].contiguous().to(
             device=self.cuda_device)
@@ -168,3 +192,38 @@ class IndexStaged(nn.Module):
             initial_D=EP_D.contiguous(), k=k, n_neighbors=self.n_neighbors,
             ef_search=ef_search, d_principle=self.d_principle,
             chunk_size=chunk_size)
+
+    def _search_on_device(self, query, k, ef_search):
+        """All three stages on the device: entries, subgraph traversal, refine
+        (one launch each on the current stream, no chunks), top-k copied back
+        at the end.  The rotation runs where ``query`` lives; given the same
+        rotated query the results are those of the host refine."""
+        if self.storage_full_cuda is None:
+            self.stage_refine()
+        device = self.cuda_device
+        if query.is_cuda:
+            query = torch.matmul(query, self.VT_cuda.T).contiguous()
+        else:
+            query = torch.matmul(query, self.VT.T).contiguous().to(device)
+        query_cuda = query[:, :self.d_principle].contiguous()
+        EP_I, EP_D = self.entry.search(query_cuda)
+        batch = query.size(0)
+        cand_I = torch.empty(batch, kernels.BEAM_WIDTH, ef_search,
+                             dtype=torch.long, device=device)
+        cand_D = torch.empty(batch, kernels.BEAM_WIDTH, ef_search,
+                             dtype=torch.float, device=device)
+        sub = kernels.prepare_graph(
+            self.subgraph_cuda.indptr, self.subgraph_cuda.indices,
+            self.mapping_cuda, self.storage_cuda.size(0), self.n_neighbors)
+        full = kernels.prepare_full_graph(self.fullgraph_cuda.indptr,
+                                          self.fullgraph_cuda.indices)
+        kernels.traverse_prepared(cand_I, cand_D, sub, self.storage_cuda,
+                                  query_cuda, EP_I.contiguous(),
+                                  EP_D.contiguous())
+        cand_I, cand_D = cand_I.flatten(1), cand_D.flatten(1)
+        topk_I = torch.empty(batch, k, dtype=torch.long, device=device)
+        topk_D = torch.empty(batch, k, dtype=torch.float, device=device)
+        kernels.traverse_refine_cuda(
+            topk_I, topk_D, cand_I, cand_D, cand_I, cand_D, sub, full,
+            self.storage_full_cuda, query, ef_search, self.d_principle)
+        return topk_I.cpu(), topk_D.cpu()

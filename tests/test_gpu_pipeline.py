@@ -10,7 +10,7 @@ import torch
 
 import oracle
 from pilotann_amd import kernels, layers, utils
-from common import Problem
+from common import Problem, assert_same_search
 
 pytestmark = pytest.mark.gpu
 
@@ -97,6 +97,14 @@ def test_index_staged_end_to_end(device):
     # chunking does not change the answer
     again_I, again_D = index.search(q, k=k, ef_search=32, chunk_size=512)
     assert torch.equal(again_I, top_I) and torch.equal(again_D, top_D)
+    # the refine on the device gives the host refine's answer (same rotated
+    # query: a host query is rotated on the host in both)
+    dev_I, dev_D = index.search(q, k=k, ef_search=32, refine='device')
+    assert not dev_I.is_cuda
+    assert_same_search(dev_I.numpy(), dev_D.numpy(), top_I.numpy(), top_D.numpy())
+    # a device query is rotated there: another matrix product, same quality
+    gpu_I, gpu_D = index.search(q.to(device), k=k, ef_search=32, refine='device')
+    assert abs(utils.recall(gpu_I, target) - utils.recall(top_I, target)) < 0.005
     # a reloaded checkpoint searches identically
     import io
     blob = io.BytesIO()

@@ -62,8 +62,9 @@ def run_both(p, dp, ef_search, k, cand_I, cand_D, device, n_buffers=None,
     out_D = torch.empty(B, k, dtype=torch.float, device=device)
     counters = torch.zeros(6, dtype=torch.long, device=device)
     kernels.traverse_refine_cuda(out_I, out_D, buf_I, buf_D, init_I, init_D,
-                                 sub, full, p.x.to(device), p.query.to(device),
-                                 ef_search, dp, counters=counters)
+                                 sub, full, kernels.prepare_rows(p.x.to(device)),
+                                 p.query.to(device), ef_search, dp,
+                                 counters=counters)
     torch.cuda.synchronize()
     got = dict(out_I=out_I.cpu().numpy(), out_D=out_D.cpu().numpy(),
                buf_I=buf_I.cpu().numpy(), buf_D=buf_D.cpu().numpy(),
@@ -79,6 +80,7 @@ def run_both(p, dp, ef_search, k, cand_I, cand_D, device, n_buffers=None,
     (128, 32, 24, 32, 64, 20, 'nsw'),
     (96, 40, 32, 16, 100, 100, 'nsg'),    # odd number of groups before the tail
     (768, 128, 32, 16, 64, 10, 'nsw'),    # long rows
+    (256, 40, 32, 16, 32, 10, 'nsw'),     # odd first group, batched loads, rest
     (64, 16, 48, 64, 300, 10, 'nsw'),     # heap tail in LDS
 ])
 def test_refine_matches_oracle(d, dp, deg, ef, ef_search, k, graph, device):
@@ -137,13 +139,32 @@ def test_unused_candidates_and_small_batches(device):
     sub = kernels.prepare_graph(p.sub_indptr.to(device), p.sub_indices.to(device),
                                 p.mapping.to(device), p.nodelist.numel(), p.deg)
     full = kernels.prepare_full_graph(p.indptr.to(device), p.indices.to(device))
+    rows = kernels.prepare_rows(p.x.to(device))
     empty_I = torch.empty(0, 10, dtype=torch.long, device=device)
     empty_D = torch.empty(0, 10, dtype=torch.float, device=device)
     kernels.traverse_refine_cuda(
         empty_I, empty_D, empty_I.clone(), empty_D.clone(), empty_I.clone(),
-        empty_D.clone(), sub, full, p.x.to(device),
+        empty_D.clone(), sub, full, rows,
         torch.empty(0, 64, device=device), 32, 32)
     with pytest.raises(RuntimeError):    # host tensors are refused
         kernels.traverse_refine_cuda(
             empty_I.cpu(), empty_D, empty_I, empty_D, empty_I, empty_D, sub,
+            full, rows, torch.empty(0, 64, device=device), 32, 32)
+    with pytest.raises(RuntimeError):    # plain rows are refused
+        kernels.traverse_refine_cuda(
+            empty_I, empty_D, empty_I, empty_D, empty_I, empty_D, sub,
             full, p.x.to(device), torch.empty(0, 64, device=device), 32, 32)
+
+
+@pytest.mark.parametrize('d', [8, 16, 24, 40, 768])
+def test_row_layout(d, device):
+    """pa_rows_prepare: within every 16 floats the pairs of the two groups of
+    eight are interleaved by lane; a last group without a partner stays."""
+    x = torch.arange(5 * d, dtype=torch.float32).reshape(5, d)
+    got = kernels.prepare_rows(x.to(device)).rows.cpu()
+    blocks = d // 16
+    want = x.clone()
+    if blocks:
+        head = x[:, :blocks * 16].reshape(5, blocks, 2, 4, 2)   # block, group, lane, pair
+        want[:, :blocks * 16] = head.permute(0, 1, 3, 2, 4).reshape(5, blocks * 16)
+    assert torch.equal(got, want)
