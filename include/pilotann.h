@@ -78,6 +78,21 @@ int pa_graph_prepare(const int64_t *indptr, const int64_t *indices,
                      int64_t n_storage, int n_neighbors, int32_t *adj,
                      int32_t *gid, int32_t *status, void *stream);
 
+/*
+ * Builds the device layout of vector rows, once per index: copies plain rows
+ * src [n_rows * d] into dst (another buffer of the same size) such that
+ * within every 16 floats (two groups of eight) the four 8-byte pairs of the
+ * first group and those of the second are interleaved, pair a of both next to
+ * each other.  The distance kernels give lane a of a quad accumulators 2a and
+ * 2a + 1 of the reference's eight (extension/inc/distance.h:31-55); in this
+ * layout the lane reads its share of two groups with one 16-byte load and a
+ * quad covers 64 contiguous bytes per instruction.  A last group without a
+ * partner (d / 8 odd) stays as it is.  d must be a multiple of 8.
+ * Asynchronous on `stream`.
+ */
+int pa_rows_prepare(float *dst, const float *src, int64_t n_rows, int d,
+                    void *stream);
+
 /* ---- traversal ----------------------------------------------------------- */
 
 /*
@@ -101,7 +116,8 @@ int pa_traverse_plan(int64_t n_storage, int64_t batch, int dp, int ef_total,
  *         query b start at b * k, best first; unused slots hold -1 / +inf
  *         at the end.  Ids are global.
  *   adj, gid: from pa_graph_prepare.   mapping [n_nodes] int64 as there.
- *   storage [n_storage * dp] float, query [batch * dp] float.
+ *   storage [n_storage * dp] float in the layout of pa_rows_prepare,
+ *         query [batch * dp] float (plain).
  *   init_I / init_D [batch * n_init]: entry ids (global, negative = unused)
  *         and their squared distances over the same dp coordinates.
  *   counters: NULL, or 5 uint64 device words that are incremented by
@@ -179,7 +195,8 @@ int pa_traverse_refine(int64_t *out_I, float *out_D, int64_t *buf_I,
  *   topk_I / topk_D [batch * k]: host, out.
  *   full_* / sub_* : host CSR of the full graph and of the subgraph (global
  *   ids), storage [n_nodes * d_model] and query [batch * d_model]: host.
- *   adj, gid, mapping, storage_dev [n_storage * d_principle],
+ *   adj, gid, mapping, storage_dev [n_storage * d_principle] (in the layout
+ *   of pa_rows_prepare),
  *   query_dev [batch * d_principle], init_I / init_D [batch * n_init]: device.
  *   caller_stream: the stream that produced query_dev / init_*; it is
  *   synchronised before the first chunk starts (pipeline_cpu.cpp:74-75).
@@ -226,16 +243,7 @@ int pa_pipeline(int64_t *topk_I, float *topk_D, const int64_t *full_indptr,
  *   workspace: at least pa_refine_plan()'s bytes, 256-byte aligned, not
  *         shared with a call that may run at the same time.
  * Asynchronous on `stream`.
- *
- * pa_rows_prepare copies plain rows src [n_rows * d_model] into dst (another
- * buffer of the same size) in the layout the refine streams: within every 16
- * floats (two groups of eight) the four 8-byte pairs of the first group and
- * those of the second are interleaved, pair a of both next to each other, so
- * that a lane reads its share of two groups with one 16-byte load.  A last
- * group without a partner stays as it is.
  */
-int pa_rows_prepare(float *dst, const float *src, int64_t n_rows, int d_model,
-                    void *stream);
 int pa_refine_plan(int64_t n_nodes, int64_t batch, int d_model, int ef_search,
                    int *n_slots, size_t *workspace_bytes);
 int pa_refine(int64_t *out_I, float *out_D, int64_t *buf_I, float *buf_D,

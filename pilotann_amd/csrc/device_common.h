@@ -82,7 +82,8 @@ __device__ __forceinline__ int wave_max_key(int x) {
     return __builtin_amdgcn_readlane(x, kWave - 1);
 }
 
-// Squared L2 between a query held in LDS and one storage row, in the order of
+// Squared L2 between a query held in LDS and one plain row (the router's leaf
+// vectors, which stay as the caller passes them), in the order of
 // the reference's host code (extension/inc/distance.h:31-55): element j of
 // every group of eight goes to accumulator j with one FMA, the eight
 // accumulators are then added left to right.  Four adjacent lanes (a quad)
@@ -234,6 +235,42 @@ __device__ __forceinline__ float quad_square_dist_long(const float *row,
         for (; g < groups; ++g) one_group(g);
     }
     return quad_reduce(a0, a1);
+}
+
+// The whole row, for the traversal's reduced rows (same interleaved layout):
+// with a length known at compile time (DP8 groups, even) all loads of the row
+// are in flight at once, DP8 / 2 of 16 bytes per lane.
+template <int DP8>
+__device__ __forceinline__ float quad_square_dist_rows(const float *row,
+                                                       const float2 *qrun,
+                                                       int groups, int part,
+                                                       bool active) {
+    if (DP8 > 0 && DP8 % 2 == 0) {
+        float a0 = 0.f, a1 = 0.f;
+        if (active) {
+            constexpr int kBlocks = DP8 > 0 ? DP8 / 2 : 1;
+            const float4 *r4 = reinterpret_cast<const float4 *>(row) + part;
+            float4 x[kBlocks];
+#pragma unroll
+            for (int b = 0; b < kBlocks; ++b) x[b] = r4[4 * b];
+            __builtin_amdgcn_sched_barrier(0);
+            const float4 *q4 = reinterpret_cast<const float4 *>(qrun);
+#pragma unroll
+            for (int b = 0; b < kBlocks; ++b) {
+                const float4 y = q4[b];
+                const float d0 = y.x - x[b].x, d1 = y.y - x[b].y;
+                a0 = fmaf(d0, d0, a0);
+                a1 = fmaf(d1, d1, a1);
+                const float d2 = y.z - x[b].z, d3 = y.w - x[b].w;
+                a0 = fmaf(d2, d2, a0);
+                a1 = fmaf(d3, d3, a1);
+                if ((b & 1) == 1) __builtin_amdgcn_sched_barrier(0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        return quad_reduce(a0, a1);
+    }
+    return quad_square_dist_long(row, qrun, groups, 0, part, active);
 }
 
 }  // namespace pa

@@ -367,7 +367,10 @@ struct Plan {
     RefineFn fn;
 };
 
-constexpr int kMaxWavesPerCu = 20;
+#ifndef PA_REFINE_MAX_WAVES
+#define PA_REFINE_MAX_WAVES 20
+#endif
+constexpr int kMaxWavesPerCu = PA_REFINE_MAX_WAVES;
 
 int make_plan(int64_t n_nodes, int64_t batch, int d, int ef_search, Plan *p) {
     if (n_nodes <= 0 || batch < 0) return PA_E_SHAPE;

@@ -440,11 +440,9 @@ __device__ __forceinline__ void eval_rows(const float *__restrict__ storage,
     for (int base = 0; base < n; base += kRowsPerPass) {
         const int c = base + quad;
         const bool active = c < n;
-        const float2 *row = reinterpret_cast<const float2 *>(storage);
-        if (active)
-            row = reinterpret_cast<const float2 *>(
-                      storage + (size_t)cand_id[c] * (size_t)dp) + part;
-        const float s = quad_square_dist<DP8>(row, qq, dp >> 3, active);
+        const float *row = storage;
+        if (active) row = storage + (size_t)cand_id[c] * (size_t)dp;
+        const float s = quad_square_dist_rows<DP8>(row, qq, dp >> 3, part, active);
         if (active && part == 0) cand_key[c] = s;
     }
 }

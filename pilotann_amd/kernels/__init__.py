@@ -181,8 +181,10 @@ def traverse_cuda(output_I: torch.Tensor,
 def traverse_prepared(output_I, output_D, graph: PreparedGraph, storage,
                       query, initial_I, initial_D, counters=None):
     """:func:`traverse_cuda` on an already prepared graph (no checks beyond
-    the C ABI's own)."""
+    the C ABI's own).  ``storage``: plain rows (their device layout is made
+    once and cached) or :class:`PreparedRows`."""
     lib = _lib.lib()
+    storage = prepare_rows(storage).rows
     batch_size, d_model = query.shape
     ef_search = output_I.size(-1)
     beam = output_I.size(1)
@@ -381,8 +383,28 @@ class PreparedRows:
                 _stream()), 'pa_rows_prepare')
 
 
-def prepare_rows(storage: torch.Tensor) -> PreparedRows:
-    return PreparedRows(storage)
+def prepare_rows(storage) -> PreparedRows:
+    """Cached :class:`PreparedRows` of a plain ``[n, d]`` device tensor (the
+    cache holds the tensor, an in-place change of it misses); a
+    :class:`PreparedRows` is returned as it is."""
+    if isinstance(storage, PreparedRows):
+        return storage
+    _check(storage, 'storage', 2, torch.float32, True)
+    key = (storage.data_ptr(), storage._version, tuple(storage.shape),
+           str(storage.device))
+    hit = _rows_cache.get(key)
+    if hit is not None:
+        _rows_cache.move_to_end(key)
+        return hit[0]
+    rows = PreparedRows(storage)
+    _rows_cache[key] = (rows, storage)
+    while len(_rows_cache) > _ROWS_CACHE_SIZE:
+        _rows_cache.popitem(last=False)
+    return rows
+
+
+_rows_cache = OrderedDict()
+_ROWS_CACHE_SIZE = 4
 
 
 def traverse_refine_cuda(output_I: torch.Tensor,
@@ -505,6 +527,7 @@ def pipeline(graph: list,
     prepared = prepare_graph(subgraph_cuda[0], subgraph_cuda[1],
                              subgraph_cuda[2], storage_cuda.size(0),
                              n_neighbors)
+    storage_cuda = prepare_rows(storage_cuda).rows
     topk_I = torch.empty(batch_size, k, dtype=torch.int64)
     topk_D = torch.empty(batch_size, k, dtype=torch.float32)
     with torch.cuda.device(query_cuda.device):

@@ -127,7 +127,9 @@ class IndexStaged(nn.Module):
         rotation."""
         device = self.cuda_device
         assert device is not None, 'call .to(device) first'
-        self.storage_full_cuda = kernels.prepare_rows(
+        # not through the cache of prepare_rows: the plain device copy is
+        # dropped once its device layout exists
+        self.storage_full_cuda = kernels.PreparedRows(
             self.storage.to(device).contiguous())
         self.VT_cuda = self.VT.to(device)
         self.fullgraph_cuda = GraphModule(self.fullgraph.indptr,
