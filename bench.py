@@ -242,7 +242,7 @@ def main():
                                               'write 1 GiB each)'}))
         return
 
-    cfg = dict(CONFIGS[args.config])
+    cfg = dict(CONFIGS[args.config], name=args.config)
     if args.n_base:
         cfg['n'] = args.n_base
     if args.queries:
@@ -473,6 +473,8 @@ def device_refine_figures(cfg, index, stage, query, target, ef, host_top=None):
         'refine_kernel_ms': round(ms, 3),
         'refine_counters': c,
         'refine_algorithmic_bytes': int(nbytes),
+        'refine_hbm_traffic': measured_traffic(
+            f'{cfg["name"]}/n={cfg["n"]}/queries={B}/ef={ef}/refine'),
         'refine_achieved_GBps': round(nbytes / (ms * 1e-3) / 1e9, 1),
         'refine_frac_of_hbm_peak': round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
 
