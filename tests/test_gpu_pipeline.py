@@ -102,6 +102,11 @@ def test_index_staged_end_to_end(device):
     dev_I, dev_D = index.search(q, k=k, ef_search=32, refine='device')
     assert not dev_I.is_cuda
     assert_same_search(dev_I.numpy(), dev_D.numpy(), top_I.numpy(), top_D.numpy())
+    # a large batch runs as two halves on two streams: same rows
+    big_I, big_D = index.search(q.repeat(5, 1), k=k, ef_search=32, refine='device')
+    for i in range(5):
+        assert torch.equal(big_I[512 * i:512 * (i + 1)], dev_I)
+        assert torch.equal(big_D[512 * i:512 * (i + 1)], dev_D)
     # a device query is rotated there: another matrix product, same quality
     gpu_I, gpu_D = index.search(q.to(device), k=k, ef_search=32, refine='device')
     assert abs(utils.recall(gpu_I, target) - utils.recall(top_I, target)) < 0.005
