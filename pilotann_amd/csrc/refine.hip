@@ -51,6 +51,22 @@ struct RefineArgs {
 
 __global__ void reset_refine_counter(int *counter) { *counter = 0; }
 
+// Optional per-phase cycle tally for tuning builds (-DPA_PHASE_TIMERS): adds
+// eight words after the six work counters.
+#ifdef PA_PHASE_TIMERS
+#define PA_TIMER_BEGIN() unsigned long long t_mark_ = __builtin_readcyclecounter()
+#define PA_TIMER(i)                                                  \
+    do {                                                             \
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); \
+        unsigned long long t_now_ = __builtin_readcyclecounter();    \
+        phase[i] += t_now_ - t_mark_;                                \
+        t_mark_ = t_now_;                                            \
+    } while (0)
+#else
+#define PA_TIMER_BEGIN() do {} while (0)
+#define PA_TIMER(i) do {} while (0)
+#endif
+
 // Squared L2 over the coordinates [from, d) between the query (LDS) and the
 // rows listed in cand_id[0..n), written to cand_key: 16 rows per pass, four
 // lanes per row; the accumulators start at zero at `from`
@@ -89,6 +105,10 @@ __global__ void interleave_rows(const float *__restrict__ src,
                                 row_pair_slot(p >> 2, p & 3, groups)) = v;
 }
 
+// buckets of the LDS visited table: 1024 x 4 nodes (8 KB); a query marks
+// about a thousand nodes at the headline configuration
+constexpr int kRefineSeenLog2 = 10;
+
 #define PA_REFINE_OCCUPANCY(H) \
     __attribute__((amdgpu_waves_per_eu((H) <= 256 ? 4 : (H) <= 384 ? 3 : (H) <= 1024 ? 2 : 1, 8)))
 
@@ -99,7 +119,7 @@ __global__ __launch_bounds__(kWave) PA_REFINE_OCCUPANCY(H) void refine_kernel(Re
     constexpr int kHeapCells =
         OpenList<H>::kLdsCells > kSortN ? OpenList<H>::kLdsCells : kSortN;
     struct Lds {
-        uint32_t seen_cache[kSeenCache];
+        uint32_t seen_table[Visited<kRefineSeenLog2>::kWords];
         int cand_id[kWave];
         float cand_key[kWave];
         int2 heap[kHeapCells];   // open list tail; the sorts reuse it
@@ -114,10 +134,14 @@ __global__ __launch_bounds__(kWave) PA_REFINE_OCCUPANCY(H) void refine_kernel(Re
     open.cells = lds.heap;
     int *cand_id = lds.cand_id;
     float *cand_key = lds.cand_key;
-    uint32_t *seen_cache = lds.seen_cache;
     const int d = a.d;
-    const bool use_cache = a.n_nodes <= (0xffff << kSeenCacheLog2);
     uint32_t *seen = a.seen + (size_t)blockIdx.x * (size_t)a.slot_stride;
+    Visited<kRefineSeenLog2> visited;
+    visited.init(lds.seen_table, seen, a.n_nodes);
+    // the wavefront's slice of the bitmask starts at zero and is put back to
+    // zero after every query that used it
+    visited.dirty = true;
+    visited.clean(a.words_per_slot, lane);
 
     for (;;) {
         int q = 0;
@@ -126,34 +150,16 @@ __global__ __launch_bounds__(kWave) PA_REFINE_OCCUPANCY(H) void refine_kernel(Re
         if (q >= a.batch) break;
 
         unsigned n_expand0 = 0, n_expand1 = 0, n_dist = 0, n_admit = 0, n_tail = 0, n_adj = 0;
+#ifdef PA_PHASE_TIMERS
+        unsigned long long phase[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#endif
+        PA_TIMER_BEGIN();
 
-        // fresh visited slice (it serves both searches), query to LDS
-        for (int w = lane * 4; w < a.words_per_slot; w += kWave * 4)
-            *reinterpret_cast<uint4 *>(seen + w) = make_uint4(0, 0, 0, 0);
+        // empty visited set (it serves both searches), query to LDS
+        visited.reset(lane);
         for (int i = lane; i < d; i += kWave)
             qv[query_slot(i, d >> 3)] = a.query[(size_t)q * d + i];
-        for (int i = lane; i < kSeenCache; i += kWave) seen_cache[i] = 0xffffffffu;
-        // the clearing stores must have landed before the first atomic OR;
-        // only this wavefront touches the slice
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         wave_sync();
-
-        // Returns the bitmask word before the OR.  A two-way LDS table of
-        // nodes whose bit is known to be set answers for most of them: word
-        // v mod 1024 holds the 16-bit tags v / 1024 of the two nodes seen last.
-        auto test_and_set = [&](int v) -> uint32_t {
-            uint32_t before = 0xffffffffu;
-            if (v >= 0) {
-                const int cell = v & (kSeenCache - 1);
-                const uint32_t tag = (uint32_t)v >> kSeenCacheLog2;
-                const uint32_t ways = use_cache ? seen_cache[cell] : 0xffffffffu;
-                if (!use_cache || ((ways & 0xffffu) != tag && (ways >> 16) != tag)) {
-                    before = atomicOr(&seen[v >> 5], 1u << (v & 31));
-                    if (use_cache) seen_cache[cell] = (ways << 16) | tag;
-                }
-            }
-            return before;
-        };
 
         // stage 0: subgraph from the candidates (traverse_cpu.cpp:317-326);
         // stage 1: full graph from the buffer (:327-336)
@@ -172,6 +178,7 @@ __global__ __launch_bounds__(kWave) PA_REFINE_OCCUPANCY(H) void refine_kernel(Re
                                    : a.out_D + (size_t)q * a.k;
             const int n_out = stage == 0 ? a.n_buffers : a.k;
 
+            PA_TIMER(0);
             open.reset(lane);
             Results<S> res;
             res.rk = lds.res_key;
@@ -200,13 +207,14 @@ __global__ __launch_bounds__(kWave) PA_REFINE_OCCUPANCY(H) void refine_kernel(Re
                                    tail_from, lane);
                     n_tail += n;
                     wave_sync();
+                    PA_TIMER(1);
                     if (u >= 0) {
                         dist += cand_key[rank];
                         eD[i] = dist;
                     }
                     wave_sync();
                 }
-                if (u >= 0) atomicOr(&seen[u >> 5], 1u << (u & 31));
+                if (u >= 0) visited.mark(u);
                 const int cnt = min(kWave, n_ent - base);
                 for (int j = 0; j < cnt; ++j) {
                     const int uj = __builtin_amdgcn_readlane(u, j);
@@ -215,12 +223,14 @@ __global__ __launch_bounds__(kWave) PA_REFINE_OCCUPANCY(H) void refine_kernel(Re
                         __builtin_amdgcn_readlane(__float_as_int(dist), j));
                     open.template replace<true>(float_to_key(dj), uj, lane);
                 }
+                PA_TIMER(2);
             }
 
             // traverse_cpu.cpp:82-136
             for (int step = 0; step < max_iter; ++step) {
                 int uk, u;
                 open.pop(lane, uk, u);
+                PA_TIMER(3);
                 if (u < 0 || uk >= res.worst) break;
                 n_expand0 += stage == 0, n_expand1 += stage != 0;
                 int v = -1;
@@ -234,16 +244,17 @@ __global__ __launch_bounds__(kWave) PA_REFINE_OCCUPANCY(H) void refine_kernel(Re
                     v = a.full_adj[(size_t)u * deg + lane];
                 }
                 n_adj += deg;
-                const uint32_t before = test_and_set(v);
-                const bool fresh = !((before >> (v & 31)) & 1u);
+                const bool fresh = v >= 0 && visited.mark(v);
                 const unsigned long long mask = __ballot(fresh);
                 const int n = __popcll(mask);
+                PA_TIMER(4);
                 if (n == 0) continue;
                 if (fresh) cand_id[lane_rank(mask)] = v;
                 wave_sync();
                 eval_rows_from(a.storage, qv, cand_id, cand_key, n, d, 0, lane);
                 n_dist += n;
                 wave_sync();
+                PA_TIMER(5);
                 const int dk = float_to_key(lane < n ? cand_key[lane] : INFINITY);
                 const int id = lane < n ? cand_id[lane] : -1;
                 wave_sync();
@@ -262,6 +273,7 @@ __global__ __launch_bounds__(kWave) PA_REFINE_OCCUPANCY(H) void refine_kernel(Re
                     open.replace_leaf(leaf, dj, vj, lane);
                     n_admit += 1;
                 }
+                PA_TIMER(6);
             }
 
             // traverse_cpu.cpp:138-148: now the entries compete for a slot
@@ -326,7 +338,10 @@ __global__ __launch_bounds__(kWave) PA_REFINE_OCCUPANCY(H) void refine_kernel(Re
             // lanes than those that wrote it
             __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
             wave_sync();
+            PA_TIMER(7);
         }
+
+        visited.clean(a.words_per_slot, lane);
 
         if (a.counters && lane == 0) {
             atomicAdd(&a.counters[0], (unsigned long long)n_expand0);
@@ -335,6 +350,9 @@ __global__ __launch_bounds__(kWave) PA_REFINE_OCCUPANCY(H) void refine_kernel(Re
             atomicAdd(&a.counters[3], (unsigned long long)n_admit);
             atomicAdd(&a.counters[4], (unsigned long long)n_tail);
             atomicAdd(&a.counters[5], (unsigned long long)n_adj);
+#ifdef PA_PHASE_TIMERS
+            for (int i = 0; i < 8; ++i) atomicAdd(&a.counters[6 + i], phase[i]);
+#endif
         }
     }
 }

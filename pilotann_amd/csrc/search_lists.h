@@ -426,6 +426,82 @@ struct Results {
     }
 };
 
+// ---- visited set ----------------------------------------------------------------
+//
+// Exact, like the reference's per-query marks (extension/inc/bitmask.hpp).  An
+// LDS table of 2^LOG2 buckets of four 16-bit tags remembers the nodes marked:
+// node v lives in bucket v mod 2^LOG2 under the tag v / 2^LOG2 (bucket and tag
+// give v back), and nothing is ever evicted.  While a bucket has a free slot,
+// every node ever marked for it is in it: a miss means "never marked" and the
+// node is added — no memory traffic at all.  A node that finds its bucket full
+// is marked in the wavefront's slice of a pooled bitmask in device memory
+// instead (atomic OR), which is exact as well; so is every node when the tags
+// would not fit 16 bits.  Scattered atomics on a bitmask that does not stay
+// in cache cost a random memory access each way and take bandwidth from the
+// row reads; with the table they are the exception.
+// The lanes of a wavefront mark their nodes at once: a slot is claimed with
+// an LDS compare-and-swap, a lane whose swap fails looks again.
+template <int LOG2>
+struct Visited {
+    static constexpr int kBuckets = 1 << LOG2;
+    static constexpr int kWords = 2 * kBuckets;
+    uint32_t *table;  // LDS, kWords
+    uint32_t *bits;   // device memory: one bit per node, zero between queries
+    bool small;       // tags fit 16 bits (0xffff marks a free slot)
+    bool dirty;       // this lane has set a bit in `bits`
+
+    __device__ __forceinline__ void init(uint32_t *lds_words, uint32_t *slice,
+                                         int n_nodes) {
+        table = lds_words, bits = slice;
+        small = n_nodes <= (0xffff << LOG2);
+        dirty = false;
+    }
+    __device__ __forceinline__ void reset(int lane) {
+        for (int i = lane; i < kWords; i += kWave) table[i] = 0xffffffffu;
+    }
+    // marks node v (>= 0); true if it was not marked before
+    __device__ __forceinline__ bool mark(int v) {
+        if (small) {
+            const uint32_t tag = (uint32_t)v >> LOG2;
+            uint32_t *w = table + 2 * (v & (kBuckets - 1));
+            for (;;) {
+                const uint32_t w0 = __hip_atomic_load(w, __ATOMIC_RELAXED,
+                                                      __HIP_MEMORY_SCOPE_WAVEFRONT);
+                const uint32_t w1 = __hip_atomic_load(w + 1, __ATOMIC_RELAXED,
+                                                      __HIP_MEMORY_SCOPE_WAVEFRONT);
+                if ((w0 & 0xffffu) == tag || (w0 >> 16) == tag ||
+                    (w1 & 0xffffu) == tag || (w1 >> 16) == tag)
+                    return false;
+                uint32_t *slot;
+                uint32_t old, neu;
+                if ((w0 & 0xffffu) == 0xffffu)
+                    slot = w, old = w0, neu = (w0 & 0xffff0000u) | tag;
+                else if ((w0 >> 16) == 0xffffu)
+                    slot = w, old = w0, neu = (w0 & 0xffffu) | (tag << 16);
+                else if ((w1 & 0xffffu) == 0xffffu)
+                    slot = w + 1, old = w1, neu = (w1 & 0xffff0000u) | tag;
+                else if ((w1 >> 16) == 0xffffu)
+                    slot = w + 1, old = w1, neu = (w1 & 0xffffu) | (tag << 16);
+                else
+                    break;  // bucket full
+                if (atomicCAS(slot, old, neu) == old) return true;
+            }
+        }
+        dirty = true;
+        const uint32_t before = atomicOr(&bits[v >> 5], 1u << (v & 31));
+        return !((before >> (v & 31)) & 1u);
+    }
+    // after a query: the slice back to zero if any lane touched it
+    __device__ __forceinline__ void clean(int words, int lane) {
+        if (__ballot(dirty)) {
+            for (int w = lane * 4; w < words; w += kWave * 4)
+                *reinterpret_cast<uint4 *>(bits + w) = make_uint4(0, 0, 0, 0);
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            dirty = false;
+        }
+    }
+};
+
 // ---- distances ---------------------------------------------------------------
 
 // Squared L2 from the query (LDS) to the storage rows listed in cand_id[0..n),
