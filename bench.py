@@ -217,7 +217,8 @@ def main():
     ap.add_argument('--device-refine-only', action='store_true',
                     help='only measure the search with the refine on the '
                          'device and the refine kernel alone (needs --ef), '
-                         'print those figures and exit')
+                         'print those figures and exit; with --no-context '
+                         'the refine kernel alone (4 launches)')
     ap.add_argument('--copy-calibration', action='store_true',
                     help='only run a plain 1 GiB device copy five times (to '
                          'scale the FETCH_SIZE / WRITE_SIZE counters) and exit')
@@ -256,8 +257,9 @@ def main():
     if args.device_refine_only:
         if not args.ef:
             ap.error('--device-refine-only needs --ef')
-        print(json.dumps(device_refine_figures(cfg, index, stage, query,
-                                               target, args.ef)), flush=True)
+        print(json.dumps(device_refine_figures(
+            cfg, index, stage, query, target, args.ef,
+            whole_search=not args.no_context)), flush=True)
         return
 
     # pick ef: smallest of the sweep with end-to-end recall@k >= 0.90
@@ -404,7 +406,8 @@ def context_figures(line, args, cfg, index, stage, query, target, ef,
         cfg, index, stage, query, target, ef, (top_I, top_D))
 
 
-def device_refine_figures(cfg, index, stage, query, target, ef, host_top=None):
+def device_refine_figures(cfg, index, stage, query, target, ef, host_top=None,
+                          whole_search=True):
     """The whole search with the refine on the device as well
     (`IndexStaged.search(..., refine='device')`: the full-dimension rows and
     the full graph resident in HBM, one launch per stage, top-k copied back),
@@ -413,22 +416,24 @@ def device_refine_figures(cfg, index, stage, query, target, ef, host_top=None):
     B, k, dp, d, device = stage.B, cfg['k'], cfg['dp'], cfg['d'], stage.device
     kernels = stage.kernels
     index.stage_refine()
-    # same rotated query as the host path: results must agree
-    same_I, same_D = index.search(query, k=k, ef_search=ef, refine='device')
-    agree = None
-    if host_top is not None:
-        agree = {
-            'distances_identical': bool(torch.equal(same_D, host_top[1])),
-            'rows_with_identical_ids': round(float(
-                (same_I == host_top[0]).all(-1).float().mean()), 4)}
-    query_dev = query.to(device)
-    index.search(query_dev, k=k, ef_search=ef, refine='device')
-    torch.cuda.synchronize()
-    reps = 5
-    t0 = time.perf_counter()
-    for _ in range(reps):
-        top_I, _ = index.search(query_dev, k=k, ef_search=ef, refine='device')
-    t_all = (time.perf_counter() - t0) / reps
+    agree = top_I = t_all = None
+    if whole_search:
+        # same rotated query as the host path: results must agree
+        same_I, same_D = index.search(query, k=k, ef_search=ef, refine='device')
+        agree = None
+        if host_top is not None:
+            agree = {
+                'distances_identical': bool(torch.equal(same_D, host_top[1])),
+                'rows_with_identical_ids': round(float(
+                    (same_I == host_top[0]).all(-1).float().mean()), 4)}
+        query_dev = query.to(device)
+        index.search(query_dev, k=k, ef_search=ef, refine='device')
+        torch.cuda.synchronize()
+        reps = 5
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            top_I, _ = index.search(query_dev, k=k, ef_search=ef, refine='device')
+        t_all = (time.perf_counter() - t0) / reps
 
     # the refine kernel alone
     EP_I, EP_D = stage.entries()
@@ -467,8 +472,9 @@ def device_refine_figures(cfg, index, stage, query, target, ef, host_top=None):
               + B * (n_cand + k) * 8)
     return {
         'api': "IndexStaged.search(refine='device')",
-        'queries_per_s': round(B / t_all, 1),
-        'recall_at_k': round(_utils.recall(top_I, target), 4),
+        'queries_per_s': round(B / t_all, 1) if whole_search else None,
+        'recall_at_k': (round(_utils.recall(top_I, target), 4)
+                        if whole_search else None),
         'against_host_refine': agree,
         'refine_kernel_ms': round(ms, 3),
         'refine_counters': c,

@@ -105,9 +105,17 @@ __global__ void interleave_rows(const float *__restrict__ src,
                                 row_pair_slot(p >> 2, p & 3, groups)) = v;
 }
 
-// buckets of the LDS visited table: 1024 x 4 nodes (8 KB); a query marks
-// about a thousand nodes at the headline configuration
-constexpr int kRefineSeenLog2 = 10;
+// The LDS visited table: 512 buckets of 8 nodes, 8 KB.  A query of the
+// headline configuration marks about a thousand nodes: next to no bucket fills
+// up, so most queries never touch the bitmask.  Measured per 10 000 queries:
+// 1024 x 4 5.76 ms, 2048 x 4 5.77 ms, 1024 x 8 5.52 ms, 512 x 8 5.36 ms.
+#ifndef PA_REFINE_SEEN_LOG2
+#define PA_REFINE_SEEN_LOG2 9
+#endif
+#ifndef PA_REFINE_SEEN_WAYS
+#define PA_REFINE_SEEN_WAYS 8
+#endif
+typedef Visited<PA_REFINE_SEEN_LOG2, PA_REFINE_SEEN_WAYS> RefineVisited;
 
 #define PA_REFINE_OCCUPANCY(H) \
     __attribute__((amdgpu_waves_per_eu((H) <= 256 ? 4 : (H) <= 384 ? 3 : (H) <= 1024 ? 2 : 1, 8)))
@@ -119,7 +127,7 @@ __global__ __launch_bounds__(kWave) PA_REFINE_OCCUPANCY(H) void refine_kernel(Re
     constexpr int kHeapCells =
         OpenList<H>::kLdsCells > kSortN ? OpenList<H>::kLdsCells : kSortN;
     struct Lds {
-        uint32_t seen_table[Visited<kRefineSeenLog2>::kWords];
+        uint32_t seen_table[RefineVisited::kWords];
         int cand_id[kWave];
         float cand_key[kWave];
         int2 heap[kHeapCells];   // open list tail; the sorts reuse it
@@ -136,7 +144,7 @@ __global__ __launch_bounds__(kWave) PA_REFINE_OCCUPANCY(H) void refine_kernel(Re
     float *cand_key = lds.cand_key;
     const int d = a.d;
     uint32_t *seen = a.seen + (size_t)blockIdx.x * (size_t)a.slot_stride;
-    Visited<kRefineSeenLog2> visited;
+    RefineVisited visited;
     visited.init(lds.seen_table, seen, a.n_nodes);
     // the wavefront's slice of the bitmask starts at zero and is put back to
     // zero after every query that used it

@@ -429,7 +429,7 @@ struct Results {
 // ---- visited set ----------------------------------------------------------------
 //
 // Exact, like the reference's per-query marks (extension/inc/bitmask.hpp).  An
-// LDS table of 2^LOG2 buckets of four 16-bit tags remembers the nodes marked:
+// LDS table of 2^LOG2 buckets of WAYS 16-bit tags remembers the nodes marked:
 // node v lives in bucket v mod 2^LOG2 under the tag v / 2^LOG2 (bucket and tag
 // give v back), and nothing is ever evicted.  While a bucket has a free slot,
 // every node ever marked for it is in it: a miss means "never marked" and the
@@ -438,13 +438,19 @@ struct Results {
 // instead (atomic OR), which is exact as well; so is every node when the tags
 // would not fit 16 bits.  Scattered atomics on a bitmask that does not stay
 // in cache cost a random memory access each way and take bandwidth from the
-// row reads; with the table they are the exception.
+// row reads; with the table they are the exception.  (The subgraph traversal
+// keeps its smaller two-way table of recently marked rows in front of the
+// bitmask: its bitmask slices are a quarter of the size and stay in cache,
+// and the swap loop costs that kernel more than the atomics it saves —
+// measured 3.6 against 3.3 ms.)
 // The lanes of a wavefront mark their nodes at once: a slot is claimed with
 // an LDS compare-and-swap, a lane whose swap fails looks again.
-template <int LOG2>
+template <int LOG2, int WAYS = 4>
 struct Visited {
+    static_assert(WAYS % 2 == 0, "two tags per word");
     static constexpr int kBuckets = 1 << LOG2;
-    static constexpr int kWords = 2 * kBuckets;
+    static constexpr int kBucketWords = WAYS / 2;
+    static constexpr int kWords = kBucketWords * kBuckets;
     uint32_t *table;  // LDS, kWords
     uint32_t *bits;   // device memory: one bit per node, zero between queries
     bool small;       // tags fit 16 bits (0xffff marks a free slot)
@@ -459,37 +465,50 @@ struct Visited {
     __device__ __forceinline__ void reset(int lane) {
         for (int i = lane; i < kWords; i += kWave) table[i] = 0xffffffffu;
     }
-    // marks node v (>= 0); true if it was not marked before
-    __device__ __forceinline__ bool mark(int v) {
+    // Marks node v (>= 0).  Returns 0: it was marked before; 1: it was not;
+    // 2: the bitmask was asked, `before` will hold its word as it was (the
+    // caller may look at it later, so that the atomic's round trip overlaps
+    // other work): fresh() tells.
+    __device__ __forceinline__ int probe(int v, uint32_t &before) {
         if (small) {
             const uint32_t tag = (uint32_t)v >> LOG2;
-            uint32_t *w = table + 2 * (v & (kBuckets - 1));
+            uint32_t *w = table + kBucketWords * (v & (kBuckets - 1));
             for (;;) {
-                const uint32_t w0 = __hip_atomic_load(w, __ATOMIC_RELAXED,
-                                                      __HIP_MEMORY_SCOPE_WAVEFRONT);
-                const uint32_t w1 = __hip_atomic_load(w + 1, __ATOMIC_RELAXED,
-                                                      __HIP_MEMORY_SCOPE_WAVEFRONT);
-                if ((w0 & 0xffffu) == tag || (w0 >> 16) == tag ||
-                    (w1 & 0xffffu) == tag || (w1 >> 16) == tag)
-                    return false;
-                uint32_t *slot;
-                uint32_t old, neu;
-                if ((w0 & 0xffffu) == 0xffffu)
-                    slot = w, old = w0, neu = (w0 & 0xffff0000u) | tag;
-                else if ((w0 >> 16) == 0xffffu)
-                    slot = w, old = w0, neu = (w0 & 0xffffu) | (tag << 16);
-                else if ((w1 & 0xffffu) == 0xffffu)
-                    slot = w + 1, old = w1, neu = (w1 & 0xffff0000u) | tag;
-                else if ((w1 >> 16) == 0xffffu)
-                    slot = w + 1, old = w1, neu = (w1 & 0xffffu) | (tag << 16);
-                else
-                    break;  // bucket full
-                if (atomicCAS(slot, old, neu) == old) return true;
+                uint32_t word[kBucketWords];
+#pragma unroll
+                for (int i = 0; i < kBucketWords; ++i)
+                    word[i] = __hip_atomic_load(w + i, __ATOMIC_RELAXED,
+                                                __HIP_MEMORY_SCOPE_WAVEFRONT);
+                bool found = false;
+                int at = -1;  // first free slot: word at / 2, half at % 2
+#pragma unroll
+                for (int i = kBucketWords - 1; i >= 0; --i) {
+                    found |= (word[i] & 0xffffu) == tag || (word[i] >> 16) == tag;
+                    at = (word[i] >> 16) == 0xffffu ? 2 * i + 1 : at;
+                    at = (word[i] & 0xffffu) == 0xffffu ? 2 * i : at;
+                }
+                if (found) return 0;
+                if (at < 0) break;  // bucket full
+                uint32_t old = word[0];
+#pragma unroll
+                for (int i = 1; i < kBucketWords; ++i) old = (at >> 1) == i ? word[i] : old;
+                const uint32_t neu = (at & 1) ? (old & 0xffffu) | (tag << 16)
+                                              : (old & 0xffff0000u) | tag;
+                if (atomicCAS(w + (at >> 1), old, neu) == old) return 1;
             }
         }
         dirty = true;
-        const uint32_t before = atomicOr(&bits[v >> 5], 1u << (v & 31));
-        return !((before >> (v & 31)) & 1u);
+        before = atomicOr(&bits[v >> 5], 1u << (v & 31));
+        return 2;
+    }
+    __device__ __forceinline__ static bool fresh(int state, uint32_t before, int v) {
+        return state == 1 || (state == 2 && !((before >> (v & 31)) & 1u));
+    }
+    // marks node v (>= 0); true if it was not marked before
+    __device__ __forceinline__ bool mark(int v) {
+        uint32_t before = 0;
+        const int state = probe(v, before);
+        return fresh(state, before, v);
     }
     // after a query: the slice back to zero if any lane touched it
     __device__ __forceinline__ void clean(int words, int lane) {
