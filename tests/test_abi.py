@@ -44,3 +44,33 @@ def test_host_only_entry_points():
                                4, 100, 60, 8, 10, 16) == -3
     assert lib.pa_pipeline(*([None] * 15), 100, 1000, 250, 64, 32, 32, 32, 16,
                            10, 30, None) == -9
+
+
+def test_device_refine_argument_errors_on_the_host():
+    """pa_rows_prepare / pa_refine reject bad sizes before any device call;
+    the Python wrappers refuse host tensors and plain rows."""
+    import pytest
+    import torch
+    from pilotann_amd import kernels
+    lib = _lib.lib()
+    assert lib.pa_rows_prepare(None, None, 10, 60, None) == -3
+    assert lib.pa_rows_prepare(None, None, -1, 64, None) == -2
+    assert lib.pa_rows_prepare(None, None, 0, 64, None) == 0
+    assert lib.pa_rows_prepare(None, None, 10, 64, None) == -1
+    def refine(batch=4, n_nodes=100, d=64, dp=32, n_init=8, n_buf=8, k=5, ef=16,
+               sub_deg=32, full_deg=32):
+        return lib.pa_refine(*([None] * 12), batch, n_nodes, d, dp, n_init, n_buf,
+                             k, ef, sub_deg, full_deg, None, 0, None, None)
+    assert refine(batch=-1) == -2
+    assert refine(n_nodes=1 << 31) == -10
+    assert refine(sub_deg=0) == -4
+    assert refine(full_deg=65) == -4
+    assert refine(dp=12) == -3
+    assert refine(dp=72) == -3
+    x = torch.zeros(4, 64)
+    with pytest.raises(RuntimeError):
+        kernels.PreparedRows(x)
+    ids, dist = torch.zeros(4, 8, dtype=torch.long), torch.zeros(4, 8)
+    with pytest.raises(RuntimeError):
+        kernels.traverse_refine_cuda(ids, dist, ids, dist, ids, dist, None, None,
+                                     x, x, 16, 32)
