@@ -1,7 +1,8 @@
 // Device-side lists of the per-query search, shared by the subgraph traversal
 // and the full-dimension refine (gfx950, one 64-lane wavefront per query): the
 // open list (the reference's array heap, extension/inc/heapq.cuh:13-88, top
-// levels in registers), the result list, and the batched row distances.
+// levels in registers), the result list, the exact visited table of the refine,
+// and the batched row distances.
 #ifndef PILOTANN_SEARCH_LISTS_H
 #define PILOTANN_SEARCH_LISTS_H
 

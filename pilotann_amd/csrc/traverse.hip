@@ -16,8 +16,9 @@
 //     rows already known to be marked;
 //   * a distance is the reference's eight-accumulator FMA sum
 //     (extension/inc/distance.h:31-55) bit for bit: four lanes share a row,
-//     lane a of the quad owns accumulators 2a and 2a+1 and streams its 8
-//     bytes of every 32-byte group.
+//     lane a of the quad owns accumulators 2a and 2a+1 and streams its 16
+//     bytes of every 64-byte block of the row (rows are in the layout of
+//     pa_rows_prepare: the pairs of two groups of eight interleaved by lane).
 // Expansion of a node therefore costs one coalesced row of neighbour ids, an
 // atomic for each neighbour the LDS table does not know and one coalesced
 // 4*dp-byte row per unvisited neighbour, 16 rows in flight per pass.
