@@ -119,3 +119,53 @@ def test_random_refine(seed, device):
         assert np.array_equal(init_D.cpu().numpy(), ref_init_D)
     assert_same_search(buf_I.cpu().numpy(), buf_D.cpu().numpy(), ref_buf_I, ref_buf_D)
     assert_same_search(out_I.cpu().numpy(), out_D.cpu().numpy(), ref_I, ref_D)
+
+
+def test_full_buckets_and_reused_wavefronts(device):
+    """Many marks per query on a graph of 50 000 nodes: buckets of the LDS
+    visited table fill up and the device bitmask takes over; more queries than
+    resident wavefronts, so a wavefront starts its next query after one that
+    used its bitmask slice."""
+    n, n_sub, d, dp, deg, ef_search, n_init, k, B = 50_000, 20_000, 16, 8, 32, 128, 64, 10, 7000
+    g = torch.Generator().manual_seed(77)
+    nodelist = torch.randperm(n, generator=g)[:n_sub].sort().values
+    mapping = torch.full((n,), -1, dtype=torch.long)
+    mapping[nodelist] = torch.arange(n_sub)
+    sub = random_rows(g, n_sub, n_sub, nodelist, deg)
+    rowlen = torch.zeros(n, dtype=torch.long)
+    rowlen[nodelist] = deg
+    sub_indptr = torch.zeros(n + 1, dtype=torch.long)
+    sub_indptr[1:] = torch.cumsum(rowlen, 0)
+    full = random_rows(g, n, n, torch.arange(n), deg)
+    full_indptr = torch.arange(n + 1, dtype=torch.long) * deg
+    x = torch.randn(n, d, generator=g)
+    query = torch.randn(B, d, generator=g)
+    cand = nodelist[torch.randint(n_sub, (B, n_init), generator=g)].contiguous()
+    xn, qn = x.numpy(), query.numpy()
+    cand_D = torch.from_numpy(np.stack([
+        oracle.square_dist(np.ascontiguousarray(qn[b, :dp]),
+                           np.ascontiguousarray(xn[:, :dp]), cand[b].numpy().copy())
+        for b in range(B)]))
+    ref_buf_I, ref_buf_D = cand.numpy().copy(), cand_D.numpy().copy()
+    ref_I = np.empty((B, k), np.int64)
+    ref_D = np.empty((B, k), np.float32)
+    oracle.traverse_refine(ref_I, ref_D, ref_buf_I, ref_buf_D, ref_buf_I, ref_buf_D,
+                           [sub_indptr.numpy(), sub.flatten().numpy()],
+                           [full_indptr.numpy(), full.flatten().numpy()], xn, qn,
+                           ef_search, dp)
+    sub_g = kernels.prepare_graph(sub_indptr.to(device), sub.flatten().contiguous().to(device),
+                                  mapping.to(device), n_sub, deg)
+    full_g = kernels.prepare_full_graph(full_indptr.to(device),
+                                        full.flatten().contiguous().to(device), deg)
+    buf_I, buf_D = cand.to(device), cand_D.to(device)
+    out_I = torch.empty(B, k, dtype=torch.long, device=device)
+    out_D = torch.empty(B, k, dtype=torch.float, device=device)
+    counters = torch.zeros(6, dtype=torch.long, device=device)
+    kernels.traverse_refine_cuda(out_I, out_D, buf_I, buf_D, buf_I, buf_D, sub_g, full_g,
+                                 kernels.PreparedRows(x.to(device)), query.to(device),
+                                 ef_search, dp, counters=counters)
+    torch.cuda.synchronize()
+    assert_same_search(buf_I.cpu().numpy(), buf_D.cpu().numpy(), ref_buf_I, ref_buf_D)
+    assert_same_search(out_I.cpu().numpy(), out_D.cpu().numpy(), ref_I, ref_D)
+    # far more marks per query than the table's 4096 slots can hold evenly
+    assert counters[2].item() / B > 1500
