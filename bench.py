@@ -427,9 +427,10 @@ def device_refine_figures(cfg, index, stage, query, target, ef, host_top=None,
                 'rows_with_identical_ids': round(float(
                     (same_I == host_top[0]).all(-1).float().mean()), 4)}
         query_dev = query.to(device)
-        index.search(query_dev, k=k, ef_search=ef, refine='device')
+        for _ in range(3):      # the device idles during the host stages
+            index.search(query_dev, k=k, ef_search=ef, refine='device')
         torch.cuda.synchronize()
-        reps = 5
+        reps = 10
         t0 = time.perf_counter()
         for _ in range(reps):
             top_I, _ = index.search(query_dev, k=k, ef_search=ef, refine='device')

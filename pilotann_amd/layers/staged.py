@@ -120,6 +120,19 @@ class IndexStaged(nn.Module):
             kernels.prepare_graph(
                 self.subgraph_cuda.indptr, self.subgraph_cuda.indices,
                 self.mapping_cuda, self.storage_cuda.size(0), self.n_neighbors)
+            # The two streams of the device search are made and used once
+            # now, early: the runtime hands streams their hardware queue (of
+            # a few) at first use, in turn, and a pair first used later may
+            # end up sharing a queue with the stream the search is called on
+            # (the two halves of a batch then run one after the other:
+            # measured 10.9 instead of 8.8 ms per 10 000 queries).
+            if self._streams is None:
+                self._streams = [torch.cuda.Stream(device=device)
+                                 for _ in range(2)]
+                for stream in self._streams:
+                    with torch.cuda.stream(stream):
+                        torch.zeros(1, device=device)
+                    stream.synchronize()
         return self
 
     def stage_refine(self):
