@@ -131,7 +131,8 @@ __global__ __launch_bounds__(kWave) PA_REFINE_OCCUPANCY(H) void refine_kernel(Re
         int cand_id[kWave];
         float cand_key[kWave];
         int2 heap[kHeapCells];   // open list tail; the sorts reuse it
-        int res_key[S * kWave];  // result list: keys (values: the slot's memory)
+        int res_key[Results<S>::kLdsKeys];  // result list: keys, unless in registers
+                                            // (values: the slot's memory)
     };
     __shared__ __align__(16) Lds lds;
     extern __shared__ __align__(16) float qv[];  // the query, query_slot layout
@@ -316,7 +317,7 @@ __global__ __launch_bounds__(kWave) PA_REFINE_OCCUPANCY(H) void refine_kernel(Re
 #pragma unroll
             for (int s = 0; s < S; ++s) {
                 const int e = lane * S + s;
-                if (e < H) okey[e] = key_to_float(res.rk[e]), oval[e] = res.rv[e];
+                if (e < H) okey[e] = key_to_float(res.cell_key(lane, s)), oval[e] = res.rv[e];
             }
             wave_sync();
             for (int size = 2; size <= a.sort_n; size <<= 1) {

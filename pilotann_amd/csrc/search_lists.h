@@ -372,13 +372,21 @@ struct OpenList {
 // position of one cell that holds it: an insert is one store to that cell,
 // one read of every lane's own cells and a wavefront maximum.  Empty cells
 // hold +inf (so the maximum is +inf until H candidates came), cells beyond H
-// hold -inf and never win.
+// hold -inf and never win.  (Long lists keep the keys in registers instead.)
 
 template <int S>
 struct Results {
     static constexpr int kInf = 0x7f800000;      // float_to_key(+inf)
     static constexpr int kNegInf = (int)0x807fffff;  // float_to_key(-inf)
-    int *rk;      // LDS: float_to_key of the distance, kWave * S cells
+    // Long lists (eight cells per lane and more) keep their keys in
+    // registers: that is lane-masked selects instead of LDS traffic per
+    // insert, and 4 KB of LDS less per wavefront at H = 1024, which is what
+    // bounds the residency there (measured 28.1 -> 23.3 ms per 10 000 queries
+    // at H = 1024; at H = 256 the LDS form is as fast or faster).
+    static constexpr bool kRegKeys = S >= 8;
+    static constexpr int kLdsKeys = kRegKeys ? 4 : S * kWave;
+    int key_reg[S];  // kRegKeys: the lane's cells
+    int *rk;      // !kRegKeys: LDS, float_to_key of the distance, kWave * S cells
     int *rv;      // device memory: the values, same cells (written once per
                   // insert, read at the end; every lane stores the same value
                   // to a cell and so reads back its own store)
@@ -392,20 +400,34 @@ struct Results {
         for (int s = 0; s < S; ++s) {
             const int c = lane * S + s;
             const int k = c < H ? kInf : kNegInf;
-            rk[c] = k, rv[c] = -1;
+            if (kRegKeys) key_reg[s] = k;
+            else rk[c] = k;
+            rv[c] = -1;
             lane_max = max(lane_max, k);
         }
         worst = kInf;
         pos = 0;
+    }
+    __device__ __forceinline__ int cell_key(int lane, int s) const {
+        return kRegKeys ? key_reg[s] : rk[lane * S + s];
     }
     // Caller has checked k < worst.  In two parts so that the caller can put
     // independent work between the LDS traffic and its use.
     __device__ __forceinline__ void begin_insert(int k, int v, int lane, int (&key)[S]) {
         // Every lane stores the same pair to the same cell, so the lane that
         // owns the cell reads back its own store: program order is enough.
-        rk[pos] = k, rv[pos] = v;
+        rv[pos] = v;
+        if (kRegKeys) {
 #pragma unroll
-        for (int s = 0; s < S; ++s) key[s] = rk[lane * S + s];
+            for (int s = 0; s < S; ++s) {
+                key_reg[s] = lane * S + s == pos ? k : key_reg[s];
+                key[s] = key_reg[s];
+            }
+        } else {
+            rk[pos] = k;
+#pragma unroll
+            for (int s = 0; s < S; ++s) key[s] = rk[lane * S + s];
+        }
     }
     __device__ __forceinline__ void finish_insert(int lane, const int (&key)[S]) {
         int m = key[0];

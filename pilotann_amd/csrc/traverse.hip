@@ -105,8 +105,8 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
         float cand_key[kWave];
         float query[DP8 ? query_floats(8 * DP8) : 4];
         int2 heap[kHeapCells];  // open list tail; the final sort reuses it
-        int res_key[S * kWave];  // result list: keys (the values are in the slot's
-                                 // memory behind the visited slice)
+        int res_key[Results<S>::kLdsKeys];  // result list: keys, unless in registers
+                                            // (values: the slot's memory)
     };
     __shared__ __align__(16) Lds lds;
     extern __shared__ __align__(16) float query_any_length[];  // DP8 == 0 only
@@ -321,7 +321,7 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
 #pragma unroll
         for (int s = 0; s < S; ++s) {
             const int e = lane * S + s;
-            if (e < H) okey[e] = key_to_float(res.rk[e]), oval[e] = res.rv[e];
+            if (e < H) okey[e] = key_to_float(res.cell_key(lane, s)), oval[e] = res.rv[e];
         }
         wave_sync();
         for (int size = 2; size <= a.sort_n; size <<= 1) {
