@@ -27,7 +27,13 @@
  * hand-derived states; distance against float64; the search against brute
  * force on small connected graphs, and against hand-built graphs that
  * isolate each rule (iteration cap, stop at the first negative neighbour,
- * entries merged after the loop, front padding when k exceeds the heap).
+ * entries merged after the loop, front padding when k exceeds the heap, an
+ * open list of exactly 2 * HEAP_SIZE cells, the gate in front of both lists,
+ * the stop on a popped key equal to the worst kept, the two expansions of
+ * the refine's first stage, the visited marks its stages share, and what
+ * happens to equal keys in every heap primitive).  Each of these rules was
+ * also changed on purpose in a copy of this file; every such copy fails one
+ * of those tests.
  */
 #include <math.h>
 #include <stdint.h>

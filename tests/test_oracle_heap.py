@@ -122,6 +122,7 @@ def test_replace_displaces_a_live_leaf_while_cells_are_free():
     k, v = arrays(start, [10, 11, 12, 13, 14, -1, -1])
     oracle.heap_replace(k, v, 11.0, 99)   # ties lose (heapq.cuh:62)
     assert k.tolist() == start
+    assert v.tolist() == [10, 11, 12, 13, 14, -1, -1]   # 14 keeps its cell
 
 
 def test_pop_known_state():
@@ -138,8 +139,26 @@ def test_pushpop_known_state():
     assert k.tolist() == [-9, -5, -7]
     oracle.heap_pushpop(k, v, -9.0, 3)    # tie: ignored (heapq.cuh:83)
     assert k.tolist() == [-9, -5, -7]
+    assert v.tolist() == [0, 1, 2]        # the root keeps its value
     oracle.heap_pushpop(k, v, -6.0, 3)
     assert k.tolist() == [-7, -5, -6] and v.tolist() == [2, 1, 3]
+
+
+def test_equal_keys_keep_their_places():
+    """The tie rules of heapq.cuh, visible in the values only.  Sinking takes
+    the left child when both children are equal (:19-21) and stops on a child
+    equal to the sinking key (:22-24); a rising key stops under an equal
+    parent (:69-71)."""
+    k, v = arrays([1, 5, 5], [0, 1, 2])
+    assert oracle.heap_pop(k, v) == (1.0, 0)
+    assert k.tolist() == [5, INF, 5] and v.tolist() == [1, -1, 2]
+    k, v = arrays([-9, -5, -4], [0, 1, 2])
+    oracle.heap_pushpop(k, v, -5.0, 3)    # new root equals its smaller child
+    assert k.tolist() == [-5, -5, -4] and v.tolist() == [3, 1, 2]
+    k, v = arrays([1, 9, 2, 10, 11, INF, INF], [10, 11, 12, 13, 14, -1, -1])
+    oracle.heap_replace(k, v, 9.0, 99)    # leaf 11 overwritten, parent is 9 too
+    assert k.tolist() == [1, 9, 2, 10, 9, INF, INF]
+    assert v.tolist() == [10, 11, 12, 13, 99, -1, -1]
 
 
 def test_heap_size_ladder():

@@ -106,6 +106,101 @@ def test_entries_in_rising_order_can_be_lost():
     assert I == list(range(16))          # z (node 16) was never reached
 
 
+def test_open_list_has_twice_the_heap_size_cells():
+    """traverse_cpu.cpp:21-24: HEAP_SIZE = 16 result cells, 2 * 16 = 32 open
+    cells: five full levels (cells 0..30) and the lone cell 31 under cell 15.
+    Eleven entries arrive with the keys (coordinates, squared)
+    1 3 2 5 4 7 6 9 8 10 11.  Stepping heapq.cuh:47-77 by hand, every walk
+    goes left at the root and below it, because the left child is the larger
+    finite one there:
+      1 -> root; 3 -> down the empty left spine to cell 31, rises to cell 1;
+      2 -> right of the root (inf beats 3), rises to cell 2;
+      5 -> cell 1 (3 > 2), empty below: cell 31, rises to cell 3;
+      4 -> cell 1, then right (inf beats 5): rises to cell 4;
+      7 -> 1, 3 (5 > 4), empty below: rises to cell 7;   6 -> 1, 3, right: cell 8;
+      9 -> 1, 3, 7 (7 > 6), cell 15, cell 31: rises to cell 15;
+      8 -> 1, 3, 7, right (inf beats 9): cell 16, a leaf;
+      10 -> 1, 3, 7, 15 (9 > 8), its only child 31 is free: stays in cell 31;
+      11 -> 1, 3, 7, 15, 31: a leaf holding 10 <= 11: dropped.
+    With 33 cells or more cell 15 has a second, free child and 11 is kept;
+    with 31 cells or fewer cell 15 is a leaf and 10 is dropped against 9; with
+    16 cells 8 overwrites 9 in cell 15 and 10, 11 are dropped.  The entries
+    with the keys 9, 10 and 11 are the only links to the three nodes nearest
+    to the query: the first two must be found, the third must not.  All
+    entries are merged after the loop whether they were expanded or not."""
+    coords = [1, 3, 2, 5, 4, 7, 6, 9, 8, 10, 11]
+    # nodes 0..10 = the entries in this order; 11, 12, 13 = the near nodes
+    rows = [[] for _ in range(14)]
+    rows[7] = [11]            # key 9
+    rows[9] = [12]            # key 10
+    rows[10] = [13]           # key 11, dropped from the open list
+    x = points_on_axis([float(c) for c in coords] + [0.5, 0.25, 0.125])
+    q = points_on_axis([0.0])[0]
+    I, Dk = search(rows, x, q, list(range(11)),
+                   [float(c * c) for c in coords], 16, 16)
+    by_key = [0, 2, 1, 4, 3, 6, 5, 8, 7, 9, 10]      # entries, nearest first
+    assert I == [12, 11] + by_key + [-1] * 3
+    assert Dk == ([0.0625, 0.25] + [float(c * c) for c in range(1, 12)]
+                  + [INF] * 3)
+
+
+def test_candidates_not_better_than_the_worst_kept_stay_out_of_the_open_list():
+    """traverse_cpu.cpp:25-39: a distance >= the worst kept result skips the
+    result heap *and* the open list.  Such a node could never be expanded (a
+    popped key >= worst kept ends the search), so the rule shows only through
+    the cell the node would occupy.  Heap of 16, open list of 32 cells.
+    A chain a0 -> a1 -> ... -> a9 at coordinates 40, 30, 29, ..., 22 puts nine
+    results into the result heap and leaves the open list empty when a9 is
+    popped.  a9's row is  r1..r7 (coordinates 1..7), D (-30), Y (10), Z (-10),
+    W (8):
+      r1..r7 have rising keys: cells 0, 1, 2, 5, 6, 13, 14 (each walk follows
+      the larger child, the right spine); the result heap is now full and its
+      worst is a1 with 900;
+      D has 900 >= 900: skipped.  Y (100): walk 0, 2, 6, 14, both children
+      free: cell 29.  Z (100): cell 29 holds Y, 30 is free: cell 30.
+      W (64): at cell 14 the children tie (100, 100), the left one is taken:
+      W overwrites Y, the only link to the nearest node z.
+    The search then pops r1..r7, W, Z and runs dry: z is never seen.
+    Were D inserted, it would sit in cell 29, Y would go to 30, Z would
+    overwrite D in 29, W would overwrite Z, Y would be expanded and z found."""
+    a = [40.0] + [float(c) for c in range(30, 21, -1)]          # nodes 0..9
+    r = [float(c) for c in range(1, 8)]                         # nodes 10..16
+    coords = a + r + [-30.0, 10.0, -10.0, 8.0, 0.5]
+    D_, Y, Z, W, z = 17, 18, 19, 20, 21
+    rows = [[i + 1] for i in range(9)] + [list(range(10, 17)) + [D_, Y, Z, W]]
+    rows += [[] for _ in range(12)]
+    rows[Y] = [z]
+    x = points_on_axis(coords)
+    q = points_on_axis([0.0])[0]
+    I, Dk = search(rows, x, q, [0], [1600.0], 16, 16)
+    assert I[:8] == list(range(10, 17)) + [W]
+    assert sorted(I[8:10]) == [Y, Z]
+    assert I[10:] == [9, 8, 7, 6, 5, 4]
+    assert Dk == ([float(c * c) for c in range(1, 8)] + [64.0, 100.0, 100.0]
+                  + [float(c * c) for c in range(22, 28)])
+
+
+def test_a_popped_key_equal_to_the_worst_kept_ends_the_search():
+    """traverse_cpu.cpp:88-90: `u.key >= -buffer_D[0]` stops, equality
+    included.  Entries a (coordinate 1) and t (-16, key 256).  a's row holds
+    16 nodes at 16, 15, ..., 2 and 1.5 (falling keys: the 32-cell open list
+    keeps all of them); they fill the result heap, whose worst is then the
+    node at 16 with key 256.  The fifteen nearer ones are popped and expanded
+    (empty rows); the next pop returns a key of 256 (t or the node at 16),
+    which is not smaller than the worst kept: the search ends and t's only
+    neighbour z, the node nearest to the query, is never seen.  After the loop
+    a takes the place of the node at 16 and t loses the tie against the new
+    worst (heapq.cuh:83)."""
+    coords = [1.0, -16.0] + [float(c) for c in range(16, 1, -1)] + [1.5, 0.5]
+    z = len(coords) - 1
+    rows = [list(range(2, 18)), [z]] + [[] for _ in range(17)]
+    x = points_on_axis(coords)
+    q = points_on_axis([0.0])[0]
+    I, Dk = search(rows, x, q, [0, 1], [1.0, 256.0], 16, 16)
+    assert I == [0, 17] + list(range(16, 2, -1))
+    assert Dk == [1.0, 2.25] + [float(c * c) for c in range(2, 16)]
+
+
 def test_front_padding_when_k_exceeds_the_heap():
     """traverse_cpu.cpp:150-162 with k > HEAP_SIZE: the pops past the heap's
     16 cells return (inf, -1) and land, sign flipped, in front."""
@@ -254,3 +349,44 @@ def test_refine_stages_share_the_visited_marks():
     assert buf_I[0].tolist() == [2, 0] + [-1] * 14
     assert out_I[0].tolist() == [2, 3, 0, -1]
     assert out_D[0].tolist() == [1.0, 4.0, 16.0, INF]
+
+
+def test_refine_expands_two_nodes_on_the_subgraph():
+    """traverse_cpu.cpp:9,317-326: stage 2 runs with max_iterations =
+    REFINE_STEP = 2.  The subgraph is a chain 0 -> 1 -> 2 -> 3 -> 4 towards
+    the query: two expansions (of 0 and of 1) reach node 2 and no further, so
+    the buffer is exactly [2, 1, 0].  The full graph has no edges, stage 3 adds
+    nothing and returns the buffer's three nodes."""
+    sub = csr([[1], [2], [3], [4], []])
+    full = csr([[], [], [], [], []])
+    x = points_on_axis([5.0, 4.0, 3.0, 2.0, 1.0])
+    q = points_on_axis([0.0]).astype(np.float32)
+    out_I, out_D = np.empty((1, 4), np.int64), np.empty((1, 4), np.float32)
+    buf_I, buf_D = np.empty((1, 16), np.int64), np.empty((1, 16), np.float32)
+    oracle.traverse_refine(out_I, out_D, buf_I, buf_D,
+                           np.array([[0]], np.int64), np.array([[25.0]], np.float32),
+                           list(sub), list(full), x, q, 16, D)
+    assert buf_I[0].tolist() == [2, 1, 0] + [-1] * 13
+    assert buf_D[0].tolist() == [9.0, 16.0, 25.0] + [INF] * 13
+    assert out_I[0].tolist() == [2, 1, 0, -1]
+    assert out_D[0].tolist() == [9.0, 16.0, 25.0, INF]
+
+
+def test_stage_three_skips_what_stage_two_has_marked():
+    """traverse_cpu.cpp:317-336, the case the buffer cannot hide: with a
+    buffer of one slot stage 2 hands over node 2 only, but it has also
+    evaluated (and marked) node 3.  Stage 3 expands 2, whose row is [3, 4]:
+    3 carries the shared mark and is skipped although it is nearer than 4.
+    With a mark of its own stage 3 would return [2, 3, 4]."""
+    sub = csr([[2, 3], [], [], [], []])
+    full = csr([[], [], [3, 4], [], []])
+    x = points_on_axis([5.0, 9.0, 1.0, 2.0, 3.0])
+    q = points_on_axis([0.0]).astype(np.float32)
+    out_I, out_D = np.empty((1, 3), np.int64), np.empty((1, 3), np.float32)
+    buf_I, buf_D = np.empty((1, 1), np.int64), np.empty((1, 1), np.float32)
+    oracle.traverse_refine(out_I, out_D, buf_I, buf_D,
+                           np.array([[0]], np.int64), np.array([[25.0]], np.float32),
+                           list(sub), list(full), x, q, 16, D)
+    assert buf_I[0].tolist() == [2] and buf_D[0].tolist() == [1.0]
+    assert out_I[0].tolist() == [2, 4, -1]
+    assert out_D[0].tolist() == [1.0, 9.0, INF]
