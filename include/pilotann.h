@@ -55,7 +55,7 @@ int pa_heap_size(int ef_search);
  * (the reference re-reads indptr / indices / mapping as int64 on every
  * expansion: traverse_cuda.cu:130-140,199).
  *
- *   indptr  [n_nodes + 1], indices [indptr[n_nodes]], mapping [n_nodes]:
+ *   indptr  [n_nodes + 1], indices [nnz], mapping [n_nodes]:
  *           the int64 device arrays `traverse_cuda` receives
  *           (traverse_cuda.cu:249-258); indices are global ids, mapping is
  *           global id -> row of `storage` or -1.
@@ -69,14 +69,15 @@ int pa_heap_size(int ef_search);
  *   gid     [n_storage] int32, out: storage row -> global id.
  *   status  [1] int32 device word, out: 0, or a bit set: 1 = mapping is not
  *           a bijection onto 0..n_storage-1, 2 = a row is longer than
- *           n_neighbors, 4 = an id is >= n_nodes.
+ *           n_neighbors, 4 = an id is >= n_nodes, 8 = a row of a stored node
+ *           does not lie inside indices[0..nnz) (it is read as empty).
  *
  * Synchronises the stream and returns PA_E_GRAPH when status != 0.
  */
 int pa_graph_prepare(const int64_t *indptr, const int64_t *indices,
                      const int64_t *mapping, int64_t n_nodes,
-                     int64_t n_storage, int n_neighbors, int32_t *adj,
-                     int32_t *gid, int32_t *status, void *stream);
+                     int64_t n_storage, int64_t nnz, int n_neighbors,
+                     int32_t *adj, int32_t *gid, int32_t *status, void *stream);
 
 /*
  * Builds the device layout of vector rows, once per index: copies plain rows

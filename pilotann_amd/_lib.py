@@ -17,8 +17,8 @@ _sz = ctypes.c_size_t
 _SIGNATURES = {
     'pa_error_string': (ctypes.c_char_p, [_int]),
     'pa_heap_size': (_int, [_int]),
-    'pa_graph_prepare': (_int, [_vp, _vp, _vp, _i64, _i64, _int, _vp, _vp,
-                                _vp, _vp]),
+    'pa_graph_prepare': (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _vp,
+                                _vp, _vp, _vp]),
     'pa_traverse_plan': (_int, [_i64, _i64, _int, _int,
                                 ctypes.POINTER(_int), ctypes.POINTER(_sz)]),
     'pa_traverse': (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,

@@ -387,8 +387,8 @@ __global__ void invert_mapping(const int64_t *mapping, int64_t n_nodes,
 // One wavefront per storage row; lane i looks at entry i of the node's row.
 __global__ __launch_bounds__(256) void build_rows(
     const int64_t *indptr, const int64_t *indices, const int64_t *mapping,
-    int64_t n_nodes, int64_t n_storage, int deg, const int32_t *gid,
-    int32_t *adj, int32_t *status) {
+    int64_t n_nodes, int64_t n_storage, int64_t nnz, int deg,
+    const int32_t *gid, int32_t *adj, int32_t *status) {
     const int lane = threadIdx.x & (kWave - 1);
     const int64_t r = (int64_t)blockIdx.x * (blockDim.x / kWave) +
                       (threadIdx.x / kWave);
@@ -406,6 +406,12 @@ __global__ __launch_bounds__(256) void build_rows(
             len = deg;
         }
         if (len < 0) len = 0;
+        // a row that does not lie inside `indices` is reported and read as
+        // empty: nothing outside the array is ever touched
+        if (lo < 0 || lo > nnz || len > nnz - lo) {
+            if (lane == 0) atomicOr(status, 8);
+            len = 0;
+        }
         int64_t e = -1;
         if (lane < len) e = indices[lo + lane];
         const unsigned long long neg = __ballot(lane < len && e < 0);
@@ -569,12 +575,13 @@ extern "C" const char *pa_error_string(int code) {
 
 extern "C" int pa_graph_prepare(const int64_t *indptr, const int64_t *indices,
                                 const int64_t *mapping, int64_t n_nodes,
-                                int64_t n_storage, int n_neighbors,
-                                int32_t *adj, int32_t *gid, int32_t *status,
-                                void *stream_) {
+                                int64_t n_storage, int64_t nnz,
+                                int n_neighbors, int32_t *adj, int32_t *gid,
+                                int32_t *status, void *stream_) {
+    if (n_nodes <= 0 || n_storage <= 0 || n_storage > n_nodes || nnz < 0)
+        return PA_E_SHAPE;
     if (!indptr || !indices || !mapping || !adj || !gid || !status)
         return PA_E_NULL;
-    if (n_nodes <= 0 || n_storage <= 0 || n_storage > n_nodes) return PA_E_SHAPE;
     if (n_nodes >= (1ll << 31)) return PA_E_RANGE;
     if (n_neighbors < 1 || n_neighbors > PA_MAX_NEIGHBORS) return PA_E_NEIGHBORS;
     hipStream_t stream = (hipStream_t)stream_;
@@ -586,7 +593,7 @@ extern "C" int pa_graph_prepare(const int64_t *indptr, const int64_t *indices,
     const int rows_per_block = T / kWave;
     build_rows<<<(unsigned)((n_storage + rows_per_block - 1) / rows_per_block), T,
                  0, stream>>>(indptr, indices, mapping, n_nodes, n_storage,
-                              n_neighbors, gid, adj, status);
+                              nnz, n_neighbors, gid, adj, status);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return (int)e;
     int32_t host_status = 0;

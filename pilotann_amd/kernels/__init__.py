@@ -73,13 +73,15 @@ class PreparedGraph:
         with torch.cuda.device(dev):
             rc = _lib.lib().pa_graph_prepare(
                 _ptr(indptr), _ptr(indices), _ptr(mapping), n_nodes,
-                self.n_storage, self.n_neighbors, _ptr(self.adj),
+                self.n_storage, indices.numel(), self.n_neighbors,
+                _ptr(self.adj),
                 _ptr(self.gid), _ptr(self.status), _stream())
         if rc == -7:
             raise RuntimeError(
                 'pa_graph_prepare: malformed graph, status bits '
                 f'{int(self.status.item())} (1 mapping not a bijection, '
-                '2 row longer than n_neighbors, 4 id out of range)')
+                '2 row longer than n_neighbors, 4 id out of range, '
+                '8 row outside indices)')
         _lib.check(rc, 'pa_graph_prepare')
 
 

@@ -44,6 +44,12 @@ def test_host_only_entry_points():
                                4, 100, 60, 8, 10, 16) == -3
     assert lib.pa_pipeline(*([None] * 15), 100, 1000, 250, 64, 32, 32, 32, 16,
                            10, 30, None) == -9
+    # pa_graph_prepare: sizes first (indices of a negative length), then the
+    # pointers; the content of indptr is checked on the device
+    assert lib.pa_graph_prepare(None, None, None, 100, 50, -1, 32, None, None,
+                                None, None) == -2
+    assert lib.pa_graph_prepare(None, None, None, 100, 50, 1600, 32, None,
+                                None, None, None) == -1
 
 
 def test_device_refine_argument_errors_on_the_host():

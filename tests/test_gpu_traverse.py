@@ -230,3 +230,92 @@ def test_row_order_does_not_change_results(device):
         torch.cuda.synchronize()
         assert np.array_equal(out_I.flatten(1).cpu().numpy(), I_a)
         assert np.array_equal(out_D.flatten(1).cpu().numpy(), D_a)
+
+
+def test_rows_outside_indices_are_reported_not_read(device):
+    """A row whose start or end lies outside `indices` (a damaged checkpoint)
+    sets status bit 8 and is treated as empty; nothing outside the array is
+    read."""
+    p = Problem(n=2000, d=32, deg=32, sample_ratio=0.5, seed=4, n_query=8)
+    n_storage = p.nodelist.numel()
+    for damage in ('start beyond the end', 'negative start', 'end beyond the end'):
+        print('damaged indptr:', damage, flush=True)
+        indptr = p.sub_indptr.clone()
+        node = int(p.nodelist[n_storage // 2])
+        if damage == 'start beyond the end':
+            indptr[node] = indptr[-1] + (1 << 40)
+            indptr[node + 1] = indptr[node] + 32
+        elif damage == 'negative start':
+            indptr[node] = -(1 << 40)
+            indptr[node + 1] = indptr[node] + 32
+        else:
+            node = int(p.nodelist[-1])   # a row that straddles the end
+            indptr[node] = p.sub_indices.numel() - 16
+            indptr[node + 1:] = indptr[node] + 32
+        with pytest.raises(RuntimeError, match='status bits'):
+            kernels.PreparedGraph(indptr.to(device), p.sub_indices.to(device),
+                                  p.mapping.to(device), n_storage, 32)
+    torch.cuda.synchronize()
+
+
+def hand_built(rows, coords, entries, entry_d, ef_total, device, width=None):
+    """A search on a hand-built graph whose nodes sit on the first axis, as in
+    tests/test_oracle_traverse.py: returns the device's and the oracle's row."""
+    width = width or max(1, max(len(r) for r in rows))
+    n = len(rows)
+    indptr = torch.arange(n + 1, dtype=torch.long) * width
+    indices = torch.full((n * width,), -1, dtype=torch.long)
+    for i, r in enumerate(rows):
+        indices[i * width:i * width + len(r)] = torch.tensor(r, dtype=torch.long)
+    x = torch.zeros(n, 8)
+    x[:, 0] = torch.tensor(coords)
+    q = torch.zeros(1, 8)
+    init_I = torch.tensor([entries], dtype=torch.long)
+    init_D = torch.tensor([entry_d], dtype=torch.float)
+    ef = ef_total // 4
+    out_I = torch.empty(1, 4, ef, dtype=torch.long, device=device)
+    out_D = torch.empty(1, 4, ef, dtype=torch.float, device=device)
+    kernels.traverse_cuda(out_I, out_D, indptr.to(device), indices.to(device),
+                          torch.arange(n).to(device), x.to(device), q.to(device),
+                          init_I.to(device), init_D.to(device), width)
+    torch.cuda.synchronize()
+    ref_I = np.empty((1, ef_total), np.int64)
+    ref_D = np.empty((1, ef_total), np.float32)
+    oracle.traverse_cpu(ref_I, ref_D, init_I.numpy().copy(), init_D.numpy().copy(),
+                        indptr.numpy(), indices.numpy(), x.numpy(), q.numpy(),
+                        ef_total)
+    return (out_I.flatten().tolist(), out_D.flatten().tolist(),
+            ref_I[0].tolist(), ref_D[0].tolist())
+
+
+def test_hand_built_rules_on_the_device(device):
+    """The hand-derived cases that pin the oracle's rules
+    (tests/test_oracle_traverse.py), run on the device with the expected
+    outputs stated again: an open list of exactly 2 * 16 cells, the gate in
+    front of the open list, and the stop on a key equal to the worst kept."""
+    inf = float('inf')
+    # open list of 32 cells: the entries with keys 9 and 10 survive, 11 is dropped
+    coords = [1, 3, 2, 5, 4, 7, 6, 9, 8, 10, 11]
+    rows = [[] for _ in range(14)]
+    rows[7], rows[9], rows[10] = [11], [12], [13]
+    I, D, rI, rD = hand_built(rows, [float(c) for c in coords] + [0.5, 0.25, 0.125],
+                              list(range(11)), [float(c * c) for c in coords], 16, device)
+    assert I == [12, 11, 0, 2, 1, 4, 3, 6, 5, 8, 7, 9, 10, -1, -1, -1] == rI
+    assert D == [0.0625, 0.25] + [float(c * c) for c in range(1, 12)] + [inf] * 3 == rD
+    # a candidate tying with the worst kept stays out of the open list
+    a = [40.0] + [float(c) for c in range(30, 21, -1)]
+    r = [float(c) for c in range(1, 8)]
+    coords = a + r + [-30.0, 10.0, -10.0, 8.0, 0.5]
+    rows = [[i + 1] for i in range(9)] + [list(range(10, 17)) + [17, 18, 19, 20]]
+    rows += [[] for _ in range(12)]
+    rows[18] = [21]
+    I, D, rI, rD = hand_built(rows, coords, [0], [1600.0], 16, device)
+    assert I[:8] == list(range(10, 17)) + [20] and sorted(I[8:10]) == [18, 19]
+    assert I[10:] == [9, 8, 7, 6, 5, 4] and D == rD
+    assert sorted(I) == sorted(rI)
+    # a popped key equal to the worst kept ends the search
+    coords = [1.0, -16.0] + [float(c) for c in range(16, 1, -1)] + [1.5, 0.5]
+    rows = [list(range(2, 18)), [18]] + [[] for _ in range(17)]
+    I, D, rI, rD = hand_built(rows, coords, [0, 1], [1.0, 256.0], 16, device)
+    assert I == [0, 17] + list(range(16, 2, -1)) == rI
+    assert D == [1.0, 2.25] + [float(c * c) for c in range(2, 16)] == rD
