@@ -38,7 +38,8 @@ enum {
     PA_E_GRAPH = -7,       /* pa_graph_prepare found a malformed graph           */
     PA_E_LEAVES = -8,      /* n_leaves not a multiple of 32 (routing_cuda.cu:90) */
     PA_E_CHUNK = -9,       /* batch not a multiple of chunk (pipeline_cpu.cpp:58) */
-    PA_E_RANGE = -10       /* an id does not fit 31 bits                         */
+    PA_E_RANGE = -10,      /* an id does not fit 31 bits                         */
+    PA_E_STATIC = -11      /* index too large for pa_traverse_static's scratch   */
 };
 
 const char *pa_error_string(int code);
@@ -134,6 +135,34 @@ int pa_traverse(int64_t *out_I, float *out_D, const int32_t *adj,
                 int64_t n_nodes, int64_t n_storage, int dp, int n_init,
                 int beam, int ef, int n_neighbors, void *workspace,
                 size_t workspace_bytes, uint64_t *counters, void *stream);
+
+/*
+ * pa_traverse for callers that cannot allocate device memory (code under HIP
+ * graph capture, serving loops and harnesses that forbid it).  No counterpart
+ * in the reference.  Same arguments and same results as pa_traverse, without
+ * the workspace: the scratch is a static device array of
+ * PA_STATIC_SCRATCH_BYTES inside the library (each GPU the library runs on
+ * holds one until the process ends), and the call allocates nothing.
+ *
+ * A resident wavefront needs ceil(n_storage / 32) words rounded up to 1 KiB
+ * plus 4 bytes per cell of its result list; as many wavefronts are launched as
+ * the array holds (fewer than pa_traverse would use when the index is large,
+ * which costs time, not correctness).  PA_E_STATIC when fewer than
+ * min(batch, 256) fit: with the largest lists that is n_storage above about
+ * 4.1 million rows.
+ *
+ * All calls on one GPU share the array: calls that may overlap on one GPU
+ * (different streams, different threads) race; serialise them.  Nothing is
+ * kept between calls.
+ */
+#define PA_STATIC_SCRATCH_BYTES (128u << 20)
+int pa_traverse_static(int64_t *out_I, float *out_D, const int32_t *adj,
+                       const int32_t *gid, const int64_t *mapping,
+                       const float *storage, const float *query,
+                       const int64_t *init_I, const float *init_D,
+                       int64_t batch, int64_t n_nodes, int64_t n_storage,
+                       int dp, int n_init, int beam, int ef, int n_neighbors,
+                       uint64_t *counters, void *stream);
 
 /* ---- entry router -------------------------------------------------------- */
 

@@ -24,6 +24,9 @@ _SIGNATURES = {
     'pa_traverse': (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                            _i64, _i64, _i64, _int, _int, _int, _int, _int,
                            _vp, _sz, _vp, _vp]),
+    'pa_traverse_static': (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
+                                  _i64, _i64, _i64, _int, _int, _int, _int,
+                                  _int, _vp, _vp]),
     'pa_route': (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _int,
                         _vp]),
     'pa_traverse_cpu': (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,

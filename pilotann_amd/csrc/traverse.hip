@@ -438,6 +438,36 @@ __global__ __launch_bounds__(256) void build_rows(
     if (lane >= n_kept && lane < deg) out[lane] = -1;
 }
 
+// ---- scratch for callers that cannot allocate -----------------------------------
+//
+// pa_traverse_static runs the search in this array instead of a caller's
+// workspace.  Every GPU the library is used on holds its own copy at its own
+// address; host code never uses the array's name as a pointer, only the
+// address hipGetSymbolAddress returns for the current device.
+static __device__ __align__(256) unsigned char scratch[PA_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 64;
+
+// Device address of `scratch` on the current device, looked up once per device.
+int static_scratch(unsigned char **out) {
+    static std::mutex mutex;
+    static unsigned char *known[kMaxDevices] = {};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return PA_E_RANGE;
+    std::lock_guard<std::mutex> guard(mutex);
+    if (!known[dev]) {
+        void *ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!ptr) return PA_E_NULL;
+        known[dev] = static_cast<unsigned char *>(ptr);
+    }
+    *out = known[dev];
+    return PA_OK;
+}
+
 // ---- host side --------------------------------------------------------------------
 
 int round_up(int64_t x, int64_t m) { return (int)(((x + m - 1) / m) * m); }
@@ -569,6 +599,8 @@ extern "C" const char *pa_error_string(int code) {
         case PA_E_LEAVES: return "n_leaves must be a multiple of 32";
         case PA_E_CHUNK: return "batch must be a multiple of chunk_size";
         case PA_E_RANGE: return "an id does not fit 31 bits";
+        case PA_E_STATIC:
+            return "index too large for the static scratch of pa_traverse_static";
         default: return "unknown error";
     }
 }
@@ -615,15 +647,22 @@ extern "C" int pa_traverse_plan(int64_t n_storage, int64_t batch, int dp,
     return PA_OK;
 }
 
-extern "C" int pa_traverse(int64_t *out_I, float *out_D, const int32_t *adj,
-                           const int32_t *gid, const int64_t *mapping,
-                           const float *storage, const float *query,
-                           const int64_t *init_I, const float *init_D,
-                           int64_t batch, int64_t n_nodes, int64_t n_storage,
-                           int dp, int n_init, int beam, int ef,
-                           int n_neighbors, void *workspace,
-                           size_t workspace_bytes, uint64_t *counters,
-                           void *stream_) {
+namespace {
+
+// Checks and launch shared by pa_traverse and pa_traverse_static.  With
+// `fit_slots` the number of wavefronts is lowered to what the workspace holds
+// (at least min(batch, kMinStaticSlots), else PA_E_STATIC); without it a
+// workspace smaller than the plan's is an error.
+constexpr int kMinStaticSlots = 256;
+
+int launch_traverse(int64_t *out_I, float *out_D, const int32_t *adj,
+                    const int32_t *gid, const int64_t *mapping,
+                    const float *storage, const float *query,
+                    const int64_t *init_I, const float *init_D, int64_t batch,
+                    int64_t n_nodes, int64_t n_storage, int dp, int n_init,
+                    int beam, int ef, int n_neighbors, void *workspace,
+                    size_t workspace_bytes, bool fit_slots, uint64_t *counters,
+                    void *stream_) {
     if (batch < 0 || n_nodes <= 0 || n_init < 0 || beam < 1 || ef < 1)
         return PA_E_SHAPE;
     if (n_nodes >= (1ll << 31) || batch >= (1ll << 31)) return PA_E_RANGE;
@@ -636,7 +675,17 @@ extern "C" int pa_traverse(int64_t *out_I, float *out_D, const int32_t *adj,
     if (!out_I || !out_D || !adj || !gid || !mapping || !storage || !query ||
         !workspace || (n_init > 0 && (!init_I || !init_D)))
         return PA_E_NULL;
-    if (workspace_bytes < p.workspace_bytes) return PA_E_WORKSPACE;
+    if (fit_slots) {
+        const size_t slot_bytes = (size_t)p.slot_stride * 4;
+        const size_t fit = workspace_bytes < kWorkCounterBytes
+                               ? 0
+                               : (workspace_bytes - kWorkCounterBytes) / slot_bytes;
+        const int64_t need = batch < kMinStaticSlots ? batch : kMinStaticSlots;
+        if ((int64_t)fit < need) return PA_E_STATIC;
+        if ((size_t)p.n_slots > fit) p.n_slots = (int)fit;
+    } else if (workspace_bytes < p.workspace_bytes) {
+        return PA_E_WORKSPACE;
+    }
     if (reinterpret_cast<uintptr_t>(workspace) % 256) return PA_E_WORKSPACE;
 
     TraverseArgs a;
@@ -661,4 +710,41 @@ extern "C" int pa_traverse(int64_t *out_I, float *out_D, const int32_t *adj,
     reset_work_counter<<<1, 1, 0, stream>>>(a.work_counter);
     p.fn<<<p.n_slots, kWave, p.lds_bytes, stream>>>(a);
     return (int)hipGetLastError();
+}
+
+}  // namespace
+
+extern "C" int pa_traverse(int64_t *out_I, float *out_D, const int32_t *adj,
+                           const int32_t *gid, const int64_t *mapping,
+                           const float *storage, const float *query,
+                           const int64_t *init_I, const float *init_D,
+                           int64_t batch, int64_t n_nodes, int64_t n_storage,
+                           int dp, int n_init, int beam, int ef,
+                           int n_neighbors, void *workspace,
+                           size_t workspace_bytes, uint64_t *counters,
+                           void *stream_) {
+    return launch_traverse(out_I, out_D, adj, gid, mapping, storage, query,
+                           init_I, init_D, batch, n_nodes, n_storage, dp,
+                           n_init, beam, ef, n_neighbors, workspace,
+                           workspace_bytes, false, counters, stream_);
+}
+
+extern "C" int pa_traverse_static(int64_t *out_I, float *out_D,
+                                  const int32_t *adj, const int32_t *gid,
+                                  const int64_t *mapping, const float *storage,
+                                  const float *query, const int64_t *init_I,
+                                  const float *init_D, int64_t batch,
+                                  int64_t n_nodes, int64_t n_storage, int dp,
+                                  int n_init, int beam, int ef, int n_neighbors,
+                                  uint64_t *counters, void *stream_) {
+    unsigned char *ws = nullptr;
+    const int rc = static_scratch(&ws);
+    if (rc != PA_OK) return rc;
+    // The work counter is set by a kernel, the visited slices and the result
+    // values are cleared by the search itself, per query: nothing of an
+    // earlier call is read.
+    return launch_traverse(out_I, out_D, adj, gid, mapping, storage, query,
+                           init_I, init_D, batch, n_nodes, n_storage, dp,
+                           n_init, beam, ef, n_neighbors, ws,
+                           PA_STATIC_SCRATCH_BYTES, true, counters, stream_);
 }
