@@ -9,12 +9,19 @@ then `traverse_cuda`, inputs resident in HBM, at the smallest ef of the sweep
 whose end-to-end recall@10 (after the host refine) reaches 0.90.  One JSON
 line is printed; `value` is queries per second of that step.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
-                    [--n-base N] [--queries B] [--ef EF] [--no-cpu-baseline]
-                    [--no-context] [--copy-calibration]
+`value` is the rate of the GPU search stage alone (what this build replaces);
+the rates of the whole search at the same recall, with the refine on the host
+and on the device, are the top-level fields `end_to_end_qps_host_refine` and
+`end_to_end_qps_device_refine`.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1..c5]
+                    [--n-base N] [--queries B] [--ef EF] [--decay X] [--curve]
+                    [--no-cpu-baseline] [--no-context] [--copy-calibration]
 """
 import argparse
 import contextlib
+import glob
+import hashlib
 import json
 import os
 import sys
@@ -30,6 +37,11 @@ METRIC = 'QPS @ recall@10>=0.90 (1M x 768 fp32, 1 GPU); traversal HBM GB/s'
 HBM_PEAK_GBS = 8000.0
 
 CONFIGS = {
+    # the plumbing case: isotropic mixture as written, NSG rows, fixed random
+    # entries, 1024 queries at ef = 64
+    'c1': dict(n=100_000, d=96, dp=32, n_centers=64, sigma=0.3, decay=0.0,
+               normalize=False, ratio=0.25, graph='nsg32', entry='random32',
+               queries=1024, k=10, ef_sweep=[64], seed=101),
     # the configuration the metric is quoted on
     'c3': dict(n=1_000_000, d=768, dp=128, n_centers=1024, sigma=1.0,
                decay=0.5, normalize=True, ratio=0.25, graph='nsw64',
@@ -45,37 +57,106 @@ CONFIGS = {
                decay=0.5, normalize=False, ratio=0.25, graph='nsw32',
                entry='router32x32', queries=10_000, k=10,
                ef_sweep=[8, 16, 32, 64, 128], seed=201),
+    # the memory-bounded case: 10M x 768, 2.5M reduced rows and their graph
+    # on the device.  Only the device stage is built: the subgraph on a seeded
+    # random quarter of the nodes (the reference's sampler walks the full
+    # graph, whose 10M-node build is out of reach of a benchmark run) and no
+    # full graph, hence no refine and no end-to-end recall; the recall
+    # reported is that of the candidate lists.
+    'c5': dict(n=10_000_000, d=768, dp=128, n_centers=4096, sigma=1.0,
+               decay=0.5, normalize=True, ratio=0.25, graph='nsg48',
+               entry='router64x64', queries=10_000, k=10, ef_sweep=[128],
+               seed=501, stage_only=True, device_rng=True),
 }
+# every ef of a configuration that is timed besides the chosen one
+ALSO_TIMED = {'c4': [256, 512]}
 
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+def kernel_sources_sha16():
+    """Hash of the HIP / C++ sources the library is built from; the counter
+    figures in profiles/traffic.json carry the hash they were measured with."""
+    h = hashlib.sha256()
+    for path in sorted(glob.glob(os.path.join(ROOT, 'pilotann_amd', 'csrc', '*'))):
+        if path.endswith(('.hip', '.h', '.cpp')):
+            h.update(os.path.basename(path).encode())
+            with open(path, 'rb') as f:
+                h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def make_data(cfg, device):
+    from pilotann_amd import utils
+    kw = dict(normalize=cfg['normalize'], device=device, decay=cfg['decay'],
+              device_rng=cfg.get('device_rng', False))
+    x = utils.gaussian_mixture(cfg['n'], cfg['d'], cfg['n_centers'],
+                               cfg['sigma'], seed=cfg['seed'], **kw)
+    q = utils.gaussian_mixture(cfg['queries'], cfg['d'], cfg['n_centers'],
+                               cfg['sigma'], seed=cfg['seed'] + 1,
+                               center_seed=cfg['seed'], **kw)
+    chunk = max(64, min(1024, (1 << 31) // cfg['n']))
+    target = utils.brute_force_topk(q, x, cfg['k'], chunk=chunk).cpu()
+    return x, q, target
+
+
 def build_index(cfg, device):
-    from pilotann_amd import IndexStaged, utils
+    from pilotann_amd import IndexStaged
     t0 = time.time()
-    x = utils.gaussian_mixture(
-        cfg['n'], cfg['d'], cfg['n_centers'], cfg['sigma'], seed=cfg['seed'],
-        normalize=cfg['normalize'], device=device, decay=cfg['decay'])
-    q = utils.gaussian_mixture(
-        cfg['queries'], cfg['d'], cfg['n_centers'], cfg['sigma'],
-        seed=cfg['seed'] + 1, normalize=cfg['normalize'], device=device,
-        decay=cfg['decay'], center_seed=cfg['seed'])
-    target = utils.brute_force_topk(q, x, cfg['k']).cpu()
+    x, q, target = make_data(cfg, device)
     log(f'[bench] data + ground truth {time.time() - t0:.1f}s')
     index = IndexStaged(d_model=cfg['d'], d_principle=cfg['dp'],
                         sample_ratio=cfg['ratio'], graph_method=cfg['graph'],
                         entry_method=cfg['entry'], seed=cfg['seed'],
                         build_device=device)
     with contextlib.redirect_stdout(sys.stderr):  # keep stdout to the JSON line
-        index.train(x)
+        if cfg.get('stage_only'):
+            train_stage_only(index, x, cfg)
+        else:
+            index.train(x)
     del x
     torch.cuda.empty_cache()
     index.to(device)
     log(f'[bench] index built {time.time() - t0:.1f}s, '
         f'sampled {index.nodelist.numel()} of {cfg["n"]}')
     return index, q.cpu(), target
+
+
+def train_stage_only(index, x, cfg):
+    """What the device stage needs of `IndexStaged.train`, for a base set whose
+    full graph is out of reach of a benchmark run: rotation, a seeded random
+    sample of the nodes, the subgraph on the sample, the entry router."""
+    from pilotann_amd import utils
+    from pilotann_amd.layers.staged import GraphModule
+    n = x.size(0)
+    print('svd', index.d_principle)
+    xr, V = utils.svd(x, max_size=10_000_000, seed=index.seed)
+    index.register_buffer('VT', V.T.contiguous().cpu())
+    g = torch.Generator().manual_seed(index.seed + 1)
+    nodelist = torch.randperm(n, generator=g)[:round(index.sample_ratio * n)]
+    nodelist = nodelist.sort().values
+    mapping = torch.full((n,), -1, dtype=torch.long)
+    mapping[nodelist] = torch.arange(nodelist.numel())
+    print('build', index.graph_type, 'on', nodelist.numel(), 'sampled nodes')
+    sub = xr[nodelist.to(xr.device)]
+    sg_indptr, sg_indices = utils.graph_init(
+        sub, index.graph_type, index.n_neighbors, compute_dtype=torch.float16)
+    del sub
+    glob_ids = torch.where(sg_indices >= 0, nodelist[sg_indices.clamp(min=0)],
+                           torch.full_like(sg_indices, -1))
+    rowlen = torch.zeros(n, dtype=torch.long)
+    rowlen[nodelist] = sg_indptr[1:] - sg_indptr[:-1]
+    indptr = torch.zeros(n + 1, dtype=torch.long)
+    indptr[1:] = torch.cumsum(rowlen, 0)
+    index.register_module('subgraph', GraphModule(indptr, glob_ids))
+    index.register_buffer('nodelist', nodelist.contiguous())
+    index.register_buffer('mapping', mapping.contiguous())
+    index.register_buffer('storage', xr.cpu().contiguous())
+    del xr
+    index.fullgraph = None
+    index.entry.train(index.storage[:, :index.d_principle])
 
 
 class Stage:
@@ -119,12 +200,17 @@ class Stage:
 
 def end_to_end_recall(index, stage, ef, target, k):
     """Recall of the whole three-stage search at this ef: device candidates,
-    then the host refine on the full-dimension vectors."""
+    then the host refine on the full-dimension vectors.  Without a full
+    graph (stage-only index): the recall of the candidate lists themselves."""
     from pilotann_amd import kernels, utils
     out_I, out_D = stage.step(ef)
     torch.cuda.synchronize()
     buf_I = out_I.flatten(1).cpu()
     buf_D = out_D.flatten(1).cpu()
+    if index.fullgraph is None:
+        # share of the true nearest neighbours found among the candidates
+        hit = (buf_I.unsqueeze(-1) == target.unsqueeze(1)).any(1)
+        return float(hit.float().mean()), float('nan')
     top_I = torch.empty(stage.B, k, dtype=torch.long)
     top_D = torch.empty(stage.B, k, dtype=torch.float)
     t0 = time.perf_counter()
@@ -148,33 +234,116 @@ def algorithmic_bytes(counters, B, dp, n_init):
 
 
 def measured_traffic(key):
-    """HBM bytes per launch from the rocprofv3 counter runs summarised under
-    profiles/ (FETCH_SIZE and WRITE_SIZE, each scaled by what a plain copy of
-    known size reads on the same counter), or None for a workload that has
-    not been profiled."""
+    """Bytes per launch that left the L2 towards the fabric, from the
+    rocprofv3 counter runs summarised under profiles/ (FETCH_SIZE and
+    WRITE_SIZE, each scaled by what a plain copy of known size reads on the
+    same counter), and whether the kernel sources are still the ones those
+    runs were made with; (None, None) for a workload that has not been
+    profiled."""
     path = os.path.join(ROOT, 'profiles', 'traffic.json')
     try:
         with open(path) as f:
-            return json.load(f).get(key, {}).get('hbm_bytes_per_launch')
+            entry = json.load(f).get(key)
     except OSError:
-        return None
+        entry = None
+    if not entry:
+        return None, None
+    return (entry.get('hbm_bytes_per_launch'),
+            entry.get('kernel_sources_sha16') == kernel_sources_sha16())
 
 
-def cpu_baseline(index, stage, ef, EP_I, EP_D, budget_s=12.0):
-    """The host search of the reference (restated in oracle/) on the same
-    subgraph, reduced rows and entries, timed on this box's cores on a sample
-    of the batch sized for about `budget_s` seconds."""
+def time_stage(stage, ef, steps, warmup):
+    """Work counters of one launch (untimed), then `steps` timed passes of
+    router + traversal; the traversal alone is bracketed by events on the
+    launch stream."""
+    device = stage.device
+    EP_I, EP_D = stage.entries()
+    counters = torch.zeros(5, dtype=torch.long, device=device)
+    out_I, out_D = stage.traverse(ef, EP_I, EP_D, counters)
+    torch.cuda.synchronize()
+    counts = counters.cpu().tolist()
+    launch_bytes = algorithmic_bytes(counts, stage.B, stage.index.d_principle,
+                                     EP_I.size(1))
+    for _ in range(warmup):
+        stage.step(ef)
+    torch.cuda.synchronize()
+    ev = [(torch.cuda.Event(enable_timing=True),
+           torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    t0 = time.perf_counter()
+    for a, b in ev:
+        EP_I, EP_D = stage.entries()
+        a.record()
+        stage.traverse(ef, EP_I, EP_D)
+        b.record()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = 1e3 * elapsed / steps
+    kernel_ms = float(np.mean([a.elapsed_time(b) for a, b in ev]))
+    achieved = launch_bytes / (kernel_ms * 1e-3) / 1e9
+    return dict(ef=ef, ms_per_step=ms_per_step, kernel_ms=kernel_ms,
+                counts=counts, launch_bytes=launch_bytes, achieved=achieved,
+                out_I=out_I, out_D=out_D)
+
+
+def compare_search(I_a, D_a, I_b, D_b):
+    """Two result sets of the same searches: are the distances identical bit
+    for bit, and in how many rows do the ids differ anywhere but inside a run
+    of equal distances (where only the set has to agree)?"""
+    same_d = bool(np.array_equal(D_a, D_b))
+    rows = np.flatnonzero((I_a != I_b).any(-1))
+    outside_ties = 0
+    for r in rows:
+        if not np.array_equal(D_a[r], D_b[r]):
+            outside_ties += 1
+            continue
+        for dist in np.unique(D_a[r][I_a[r] != I_b[r]]):
+            sel = D_a[r] == dist
+            if sorted(I_a[r][sel]) != sorted(I_b[r][sel]):
+                outside_ties += 1
+                break
+    # ids that differ where the two distances differ as well: never allowed
+    wrong = int(((I_a != I_b) & (D_a != D_b)).any(-1).sum()) if not same_d else 0
+    out = dict(distances_identical=same_d,
+               rows_with_other_order_inside_ties=int(len(rows) - outside_ties),
+               rows_with_another_member_of_a_tie=int(outside_ties - wrong),
+               rows_with_id_mismatch=wrong)
+    if outside_ties and same_d:
+        # a row in which one of several candidates at exactly the same
+        # distance was kept by one search and another by the other
+        for r in rows:
+            pos = np.flatnonzero(I_a[r] != I_b[r])
+            sel = np.isin(D_a[r], D_a[r][pos])
+            if sorted(I_a[r][sel]) != sorted(I_b[r][sel]):
+                out['example'] = dict(
+                    row=int(r), positions=pos[:4].tolist(),
+                    ids_a=I_a[r][pos[:4]].tolist(), ids_b=I_b[r][pos[:4]].tolist(),
+                    distances=[float(x) for x in D_a[r][pos[:4]]])
+                break
+    return out
+
+
+def cpu_baseline(index, stage, ef, EP_I, EP_D, budget_s=8.0):
+    """The host search of the reference on the same subgraph, reduced rows and
+    entries, timed on this box's cores on whole passes over the batch for
+    about `budget_s` seconds each: the plain-C restatement in oracle/ and the
+    library's own host search (`pa_traverse_cpu`: AVX2, four rows per
+    distance call, prefetches, as traverse_cpu.cpp:92-135 has them).  The
+    faster one is reported; both return the same results."""
     import oracle
+    from pilotann_amd import kernels
     dp = index.d_principle
-    reduced = np.ascontiguousarray(index.storage[:, :dp].numpy())
-    q = np.ascontiguousarray(stage.query_rot[:, :dp].numpy())
-    indptr = index.subgraph.indptr.numpy()
-    indices = index.subgraph.indices.numpy()
+    reduced_t = index.storage[:, :dp].contiguous()
+    reduced = reduced_t.numpy()
+    q_t = stage.query_rot[:, :dp].contiguous()
+    q = q_t.numpy()
+    indptr_t, indices_t = index.subgraph.indptr, index.subgraph.indices
+    indptr, indices = indptr_t.numpy(), indices_t.numpy()
     kk = 4 * ef
-    I = EP_I.cpu().numpy()
-    D = EP_D.cpu().numpy()
+    I_t, D_t = EP_I.cpu(), EP_D.cpu()
+    I, D = I_t.numpy(), D_t.numpy()
+    B = stage.B
 
-    def run(n):
+    def run_port(n):
         out_I = np.empty((n, kk), np.int64)
         out_D = np.empty((n, kk), np.float32)
         t0 = time.perf_counter()
@@ -182,21 +351,113 @@ def cpu_baseline(index, stage, ef, EP_I, EP_D, budget_s=12.0):
                             indices, reduced, q[:n].copy(), kk)
         return time.perf_counter() - t0, out_I, out_D
 
-    run(min(stage.B, 512))  # warm-up: thread pool, page faults
-    # whole passes over the batch until the time budget is used
-    total_t, total_n, passes = 0.0, 0, 0
-    out_I = out_D = None
-    while total_t < budget_s and passes < 1000:
-        t, out_I, out_D = run(stage.B)
+    def run_avx2(n):
+        out_I = torch.empty(n, kk, dtype=torch.long)
+        out_D = torch.empty(n, kk, dtype=torch.float)
+        i, d, qq = I_t[:n].clone(), D_t[:n].clone(), q_t[:n].clone()
+        t0 = time.perf_counter()
+        kernels.traverse_cpu(out_I, out_D, i, d, indptr_t, indices_t,
+                             reduced_t, qq, kk)
+        return time.perf_counter() - t0, out_I.numpy(), out_D.numpy()
+
+    figures = {}
+    results = {}
+    for name, run in (('plain_c_port', run_port), ('avx2_host_search', run_avx2)):
+        run(min(B, 512))  # warm-up: thread pool, page faults
+        total_t, total_n, passes = 0.0, 0, 0
+        while total_t < budget_s and passes < 1000:
+            t, out_I, out_D = run(B)
+            total_t += t
+            total_n += B
+            passes += 1
+        figures[name] = dict(queries_per_s=round(total_n / total_t, 1),
+                             passes=passes, seconds=round(total_t, 1))
+        results[name] = (out_I, out_D)
+    best = max(figures, key=lambda n: figures[n]['queries_per_s'])
+    same = compare_search(*results['plain_c_port'], *results['avx2_host_search'])
+    base = dict(value=figures[best]['queries_per_s'], unit='queries/s',
+                cores=oracle.num_threads(), kind='port',
+                implementation=best,
+                sample=f'{figures[best]["passes"]} passes over the same {B}-query '
+                       f'batch (same subgraph / reduced rows / entries, '
+                       f'ef_search={kk}), {figures[best]["seconds"]}s of host search',
+                both=figures, both_agree=same['distances_identical']
+                and same['rows_with_id_mismatch'] == 0
+                and same['rows_with_another_member_of_a_tie'] == 0)
+    return base, results['plain_c_port']
+
+
+def cpu_full_graph_baseline(index, stage, EP_I, target, k, budget_s=6.0):
+    """The search without a GPU: the host search on the full graph in full
+    dimension from the same entry ids (their full-dimension distances are
+    computed on the host, inside the timed region), at the smallest ef_search
+    whose recall@k reaches 0.90 on a 2000-query sample — the role faiss' HNSW
+    plays in the reference's own table (README.md:527-534)."""
+    import oracle
+    from pilotann_amd import kernels, utils
+    if index.fullgraph is None:
+        return None
+    indptr, indices = index.fullgraph.indptr, index.fullgraph.indices
+    storage, query = index.storage, stage.query_rot
+    ids = EP_I.cpu()
+
+    def run(lo, hi, ef_search):
+        q = query[lo:hi].contiguous()
+        t0 = time.perf_counter()
+        i = ids[lo:hi].contiguous()
+        d = torch.empty(i.shape, dtype=torch.float)
+        for a in range(0, hi - lo, 500):
+            rows = storage[i[a:a + 500]]
+            d[a:a + 500] = (q[a:a + 500].unsqueeze(1) - rows).square().sum(-1)
+        out_I = torch.empty(hi - lo, k, dtype=torch.long)
+        out_D = torch.empty(hi - lo, k, dtype=torch.float)
+        kernels.traverse_cpu(out_I, out_D, i, d, indptr, indices, storage, q,
+                             ef_search)
+        return time.perf_counter() - t0, out_I
+
+    n_sample = min(2000, stage.B)
+    sweep, chosen = [], None
+    for ef_search in [e for e in (16, 24, 32, 48, 64, 96, 128, 192, 256, 384,
+                                  512, 1024) if e >= k]:
+        t, out_I = run(0, n_sample, ef_search)
+        rec = utils.recall(out_I, target[:n_sample])
+        sweep.append(dict(ef_search=ef_search, recall=round(rec, 4)))
+        if rec >= 0.90:
+            chosen = ef_search
+            break
+    if chosen is None:
+        chosen = sweep[-1]['ef_search']
+    total_t, total_n, passes, rec = 0.0, 0, 0, None
+    while total_t < budget_s and passes < 100:
+        t, out_I = run(0, stage.B, chosen)
+        rec = utils.recall(out_I, target)
         total_t += t
         total_n += stage.B
         passes += 1
-    return dict(value=total_n / total_t, unit='queries/s',
-                cores=oracle.num_threads(), kind='port',
-                sample=f'{passes} passes over the same {stage.B}-query batch '
-                       f'(same subgraph / reduced rows / entries, '
-                       f'ef_search={kk}), {total_t:.1f}s of host search'), \
-        (out_I, out_D, stage.B)
+    return dict(what='traverse_cpu (library host search, AVX2) on the full '
+                     'graph in full dimension, entry distances included',
+                ef_search=chosen, recall_at_k=round(rec, 4),
+                queries_per_s=round(total_n / total_t, 1),
+                cores=oracle.num_threads(), passes=passes, sweep=sweep)
+
+
+def stage_record(t, B, key):
+    traffic, fresh = measured_traffic(key)
+    rec = {
+        'bound': 'hbm', 'achieved': round(t['achieved'], 1),
+        'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
+        'frac': round(t['achieved'] / HBM_PEAK_GBS, 4),
+        'traffic': traffic,
+        'kernel': 'traverse_kernel',
+        'kernel_ms': round(t['kernel_ms'], 4),
+        'algorithmic_bytes_per_launch': t['launch_bytes'],
+        'counters': dict(zip(['expanded', 'adjacency_entries', 'distances',
+                              'admitted', 'result_slots'], t['counts'])),
+    }
+    if traffic is not None:
+        # the figure is a constant of a profiled run, not measured here
+        rec['traffic_kernel_sources_unchanged'] = bool(fresh)
+    return rec
 
 
 def main():
@@ -208,12 +469,18 @@ def main():
     ap.add_argument('--n-base', type=int, default=None)
     ap.add_argument('--queries', type=int, default=None)
     ap.add_argument('--ef', type=int, default=None)
+    ap.add_argument('--decay', type=float, default=None,
+                    help='exponent of the power-law spectrum of the synthetic '
+                         'data (0 = the isotropic mixture)')
+    ap.add_argument('--curve', action='store_true',
+                    help='time the stage at every ef of the sweep (no early '
+                         'stop) and report recall and rate for each')
     ap.add_argument('--no-cpu-baseline', action='store_true')
     ap.add_argument('--no-context', action='store_true',
                     help='skip the context figures (PCIe-inclusive step, '
-                         'fourfold batch, end-to-end search), so that a '
-                         'kernel trace of the run holds the timed launches '
-                         'only')
+                         'fourfold batch, end-to-end search, isotropic data), '
+                         'so that a kernel trace of the run holds the timed '
+                         'launches only')
     ap.add_argument('--device-refine-only', action='store_true',
                     help='only measure the search with the refine on the '
                          'device and the refine kernel alone (needs --ef), '
@@ -248,6 +515,8 @@ def main():
         cfg['n'] = args.n_base
     if args.queries:
         cfg['queries'] = args.queries
+    if args.decay is not None:
+        cfg['decay'] = args.decay
     device = 'cuda:0'
     torch.cuda.set_device(0)
     index, query, target = build_index(cfg, device)
@@ -268,45 +537,30 @@ def main():
     for ef in ([args.ef] if args.ef else cfg['ef_sweep']):
         rec, refine_s = end_to_end_recall(index, stage, ef, target, k)
         sweep.append(dict(ef=ef, recall=round(rec, 4),
-                          refine_qps=round(B / refine_s, 1)))
+                          refine_qps=round(B / refine_s, 1)
+                          if refine_s == refine_s else None))
         log(f'[bench] ef={ef} recall@{k}={rec:.4f} host refine {refine_s:.2f}s')
-        if rec >= 0.90:
+        if rec >= 0.90 and chosen is None:
             chosen = ef
-            break
+            if not args.curve:
+                break
     if chosen is None:
         chosen = sweep[-1]['ef']
     ef = chosen
     recall_at = [s for s in sweep if s['ef'] == ef][0]['recall']
 
-    # work counters of one launch (untimed), then the timed steps
-    EP_I, EP_D = stage.entries()
-    counters = torch.zeros(5, dtype=torch.long, device=device)
-    out_I, out_D = stage.traverse(ef, EP_I, EP_D, counters)
-    torch.cuda.synchronize()
-    counts = counters.cpu().tolist()
-    launch_bytes = algorithmic_bytes(counts, B, dp, EP_I.size(1))
-
-    for _ in range(args.warmup):
-        stage.step(ef)
-    torch.cuda.synchronize()
-    ev = [(torch.cuda.Event(enable_timing=True),
-           torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
-    t0 = time.perf_counter()
-    for a, b in ev:
-        EP_I, EP_D = stage.entries()
-        a.record()
-        stage.traverse(ef, EP_I, EP_D)
-        b.record()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms_per_step = 1e3 * elapsed / args.steps
-    kernel_ms = float(np.mean([a.elapsed_time(b) for a, b in ev]))
-    achieved = launch_bytes / (kernel_ms * 1e-3) / 1e9
+    t = time_stage(stage, ef, args.steps, args.warmup)
+    out_I, out_D = t['out_I'], t['out_D']
+    launch_bytes, ms_per_step = t['launch_bytes'], t['ms_per_step']
+    key = f'{args.config}/n={cfg["n"]}/queries={B}/ef={ef}'
 
     line = {
         'metric': METRIC,
         'value': round(B / (ms_per_step * 1e-3), 1),
         'unit': 'queries/s',
+        'value_is': 'rate of the GPU search stage (routing_cuda + '
+                    'traverse_cuda) at the ef whose end-to-end recall is '
+                    'recall_at_k; whole-search rates: end_to_end_qps_*',
         'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
         'ms_per_step': round(ms_per_step, 4),
         'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
@@ -314,26 +568,35 @@ def main():
         'config': {
             'workload': f'{args.config}: {cfg["n"]} x {cfg["d"]} '
                         f'{"unit-norm " if cfg["normalize"] else ""}'
-                        f'{cfg["n_centers"]}-component mixture, dp={dp}, '
+                        f'{cfg["n_centers"]}-component mixture '
+                        f'(sigma {cfg["sigma"]}, spectrum exponent '
+                        f'{cfg["decay"]}), dp={dp}, '
                         f'sample_ratio={cfg["ratio"]}, {cfg["graph"]}, '
                         f'{cfg["entry"]}, {B} queries, top-{k}',
             'ef': ef, 'k': k, 'recall_at_k': recall_at, 'sweep': sweep,
+            'recall_is': ('candidate lists of the device stage (no full '
+                          'graph, no refine)' if index.fullgraph is None else
+                          'whole search: device candidates, then host refine'),
             'stage': 'routing_cuda + traverse_cuda (GPU search stage)',
         },
-        'roofline': {
-            'bound': 'hbm', 'achieved': round(achieved, 1),
-            'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
-            'frac': round(achieved / HBM_PEAK_GBS, 4),
-            'traffic': measured_traffic(
-                f'{args.config}/n={cfg["n"]}/queries={B}/ef={ef}'),
-            'kernel': 'traverse_kernel',
-            'kernel_ms': round(kernel_ms, 4),
-            'algorithmic_bytes_per_launch': launch_bytes,
-            'counters': dict(zip(['expanded', 'adjacency_entries',
-                                  'distances', 'admitted', 'result_slots'],
-                                 counts)),
-        },
+        'roofline': stage_record(t, B, key),
     }
+    others = [e for e in (cfg['ef_sweep'] if args.curve else
+                          ALSO_TIMED.get(args.config, []))
+              if e != ef and not args.ef]
+    if others:
+        recalls = {s['ef']: s['recall'] for s in sweep}
+        line['config']['other_ef'] = []
+        for e in others:
+            if e not in recalls:
+                recalls[e] = round(end_to_end_recall(index, stage, e, target, k)[0], 4)
+            o = time_stage(stage, e, max(3, args.steps // 2), 1)
+            rec = stage_record(o, B, f'{args.config}/n={cfg["n"]}/queries={B}/ef={e}')
+            line['config']['other_ef'].append(dict(
+                ef=e, recall_at_k=recalls[e],
+                queries_per_s=round(B / (o['ms_per_step'] * 1e-3), 1),
+                ms_per_step=round(o['ms_per_step'], 4), roofline=rec))
+            log(f'[bench] ef={e}: {o["kernel_ms"]:.3f} ms, frac {rec["frac"]}')
     if not args.no_context:
         context_figures(line, args, cfg, index, stage, query, target, ef,
                         launch_bytes, out_D)
@@ -341,10 +604,16 @@ def main():
     if not args.no_cpu_baseline:
         EP_I, EP_D = stage.entries()
         torch.cuda.synchronize()
-        base, (ref_I, ref_D, n) = cpu_baseline(index, stage, ef, EP_I, EP_D)
+        base, (ref_I, ref_D) = cpu_baseline(index, stage, ef, EP_I, EP_D)
         line['cpu_baseline'] = base
-        same = (np.array_equal(out_D.flatten(1)[:n].cpu().numpy(), ref_D))
-        line['config']['matches_cpu_baseline'] = bool(same)
+        # the whole batch against the oracle: distances bit for bit, ids
+        # except inside runs of equal distances
+        line['config']['matches_cpu_baseline'] = compare_search(
+            out_I.flatten(1).cpu().numpy(), out_D.flatten(1).cpu().numpy(),
+            ref_I, ref_D)
+        full = cpu_full_graph_baseline(index, stage, EP_I, target, k)
+        if full:
+            line['cpu_baseline']['without_gpu'] = full
     print(json.dumps(line), flush=True)
 
 
@@ -352,8 +621,8 @@ def context_figures(line, args, cfg, index, stage, query, target, ef,
                     launch_bytes, out_D):
     """Not part of `value`: the same step with its inputs and outputs
     crossing PCIe (pageable host memory), the launch over a fourfold batch,
-    and the whole three-stage search (`IndexStaged.search`: rotation on the
-    host, entries, pipeline)."""
+    the whole three-stage search (`IndexStaged.search`: rotation on the
+    host, entries, pipeline), and the headline workload's isotropic twin."""
     B, k, dp, device = stage.B, cfg['k'], cfg['dp'], stage.device
     host_q = stage.query_rot[:, :dp].contiguous()
     torch.cuda.synchronize()
@@ -365,8 +634,8 @@ def context_figures(line, args, cfg, index, stage, query, target, ef,
     line['config']['ms_per_step_with_pcie'] = round(
         1e3 * (time.perf_counter() - t0) / 3, 3)
     # context: the same launch over four copies of the batch.  One launch
-    # keeps 5120 independent searches in flight; filling and draining them
-    # weighs less on a longer batch, which shows the kernel's marginal rate.
+    # keeps thousands of independent searches in flight; filling and draining
+    # them weighs less on a longer batch, which shows the kernel's marginal rate.
     rep = 4
     big_q = stage.query_cuda.repeat(rep, 1).contiguous()
     big_EI, big_ED = [t.repeat(rep, 1).contiguous() for t in stage.entries()]
@@ -392,18 +661,50 @@ def context_figures(line, args, cfg, index, stage, query, target, ef,
         'same_results': bool(torch.equal(big_D[-B:], out_D))}
     del big_q, big_EI, big_ED, big_I, big_D
 
-    chunk = 1000 if B % 1000 == 0 else B
-    index.search(query, k=k, ef_search=ef, chunk_size=chunk)
-    t0 = time.perf_counter()
-    top_I, top_D = index.search(query, k=k, ef_search=ef, chunk_size=chunk)
-    t_e2e = time.perf_counter() - t0
-    from pilotann_amd import utils as _utils
-    line['config']['end_to_end'] = {
-        'api': 'IndexStaged.search', 'chunk_size': chunk,
-        'queries_per_s': round(B / t_e2e, 1),
-        'recall_at_k': round(_utils.recall(top_I, target), 4)}
-    line['config']['end_to_end_device_refine'] = device_refine_figures(
-        cfg, index, stage, query, target, ef, (top_I, top_D))
+    if index.fullgraph is not None:
+        chunk = 1000 if B % 1000 == 0 else B
+        index.search(query, k=k, ef_search=ef, chunk_size=chunk)
+        t0 = time.perf_counter()
+        top_I, top_D = index.search(query, k=k, ef_search=ef, chunk_size=chunk)
+        t_e2e = time.perf_counter() - t0
+        from pilotann_amd import utils as _utils
+        line['config']['end_to_end'] = {
+            'api': 'IndexStaged.search', 'chunk_size': chunk,
+            'queries_per_s': round(B / t_e2e, 1),
+            'recall_at_k': round(_utils.recall(top_I, target), 4)}
+        line['config']['end_to_end_device_refine'] = device_refine_figures(
+            cfg, index, stage, query, target, ef, (top_I, top_D))
+        line['end_to_end_qps_host_refine'] = \
+            line['config']['end_to_end']['queries_per_s']
+        line['end_to_end_qps_device_refine'] = \
+            line['config']['end_to_end_device_refine']['queries_per_s']
+
+    if args.config == 'c3' and cfg['decay'] > 0 and not args.n_base:
+        line['config']['isotropic_mixture'] = isotropic_twin(cfg, device, args)
+
+
+def isotropic_twin(cfg, device, args):
+    """The same configuration on the isotropic mixture (every coordinate of
+    centres and noise with the same variance before the normalisation — the
+    data exactly as the configuration words it): recall of the whole search
+    and rate of the GPU stage over the configuration's ef range."""
+    iso = dict(cfg, decay=0.0)
+    index, query, target = build_index(iso, device)
+    stage = Stage(index, query, device)
+    rows = []
+    for ef in (32, 64, 128, 256):
+        rec, _ = end_to_end_recall(index, stage, ef, target, iso['k'])
+        t = time_stage(stage, ef, 5, 1)
+        rows.append(dict(ef=ef, recall_at_k=round(rec, 4),
+                         queries_per_s=round(stage.B / (t['ms_per_step'] * 1e-3), 1),
+                         kernel_ms=round(t['kernel_ms'], 4),
+                         frac=round(t['achieved'] / HBM_PEAK_GBS, 4)))
+        log(f'[bench] isotropic ef={ef} recall {rec:.4f} '
+            f'{t["kernel_ms"]:.3f} ms frac {rows[-1]["frac"]}')
+    del index, stage
+    torch.cuda.empty_cache()
+    return dict(what='same sizes, seeds and pipeline, spectrum exponent 0',
+                sweep=rows)
 
 
 def device_refine_figures(cfg, index, stage, query, target, ef, host_top=None,
@@ -481,7 +782,7 @@ def device_refine_figures(cfg, index, stage, query, target, ef, host_top=None,
         'refine_counters': c,
         'refine_algorithmic_bytes': int(nbytes),
         'refine_hbm_traffic': measured_traffic(
-            f'{cfg["name"]}/n={cfg["n"]}/queries={B}/ef={ef}/refine'),
+            f'{cfg["name"]}/n={cfg["n"]}/queries={B}/ef={ef}/refine')[0],
         'refine_achieved_GBps': round(nbytes / (ms * 1e-3) / 1e9, 1),
         'refine_frac_of_hbm_peak': round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
 
