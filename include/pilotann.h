@@ -183,6 +183,21 @@ int pa_route(int64_t *router, float *dist, const float *query,
              const float *route_vectors, const float *entry_vectors,
              int64_t batch, int n_routers, int n_leaves, int dp, void *stream);
 
+/*
+ * Replaces the query rotation of `IndexStaged.search`
+ * (pilot_ann/layers/staged.py:198-201: `query @ VT.T`, then the first
+ * d_principle coordinates for the device stage), on the matrix cores.
+ *
+ *   out   [batch * n_out] float, out: out[b][j] = sum_k query[b][k] * VT[j][k]
+ *         for j < n_out (n_out = d for the whole rotation, d_principle for
+ *         the device stage's part).
+ *   query [batch * d], VT [d * d] (row j = basis vector j), float, device.
+ * d must be a multiple of 8, 1 <= n_out <= d.  Float32 accumulation in another
+ * order than a host matmul: results agree to rounding, not bit for bit.
+ */
+int pa_rotate(float *out, const float *query, const float *VT, int64_t batch,
+              int d, int n_out, void *stream);
+
 /* ---- host stages and the chunk pipeline ------------------------------------- */
 
 /*

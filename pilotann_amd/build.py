@@ -10,7 +10,8 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, 'csrc')
 LIB = os.path.join(CSRC, 'libpilotann.so')
 
-HIP_SOURCES = ['traverse.hip', 'refine.hip', 'route.hip', 'pipeline.hip']
+HIP_SOURCES = ['traverse.hip', 'refine.hip', 'route.hip', 'rotate.hip',
+               'pipeline.hip']
 CXX_SOURCES = ['host_search.cpp']
 
 HIP_FLAGS = [

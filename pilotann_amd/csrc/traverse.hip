@@ -54,7 +54,7 @@ struct TraverseArgs {
     int *work_counter;
     unsigned long long *counters;
     int batch, n_nodes, n_storage, dp, n_init, k, H, deg, max_iter;
-    int words_per_slot, slot_stride, sort_n, lds_cells;
+    int words_per_slot, slot_stride, sort_n;
 };
 
 __global__ void reset_work_counter(int *counter) { *counter = 0; }
@@ -509,7 +509,7 @@ TraverseFn pick_kernel(int H, int dp) {
 }
 
 struct Plan {
-    int H, sort_n, lds_cells, lds_bytes, n_slots, words_per_slot, slot_stride;
+    int H, sort_n, lds_bytes, n_slots, words_per_slot, slot_stride;
     size_t workspace_bytes;
     TraverseFn fn;
 };
@@ -521,10 +521,6 @@ int make_plan(int64_t n_storage, int64_t batch, int dp, int ef_total, Plan *p) {
     if (ef_total < 1 || ef_total > PA_MAX_EF_TOTAL) return PA_E_EF;
     p->H = pa_heap_size(ef_total);
     p->sort_n = next_pow2(p->H < kWave ? kWave : p->H);
-    // LDS part of the open list (nodes 256.. of 2H, one spare), reused by the
-    // final sort of sort_n cells
-    const int tail = 2 * p->H + 2 - 256;
-    p->lds_cells = tail > p->sort_n ? tail : p->sort_n;
     // dynamic LDS: the query when its length has no specialised kernel (the
     // rest is static in the kernel)
     p->lds_bytes = (dp == 32 || dp == 64 || dp == 128) ? 0 : query_floats(dp) * 4;
@@ -704,7 +700,6 @@ int launch_traverse(int64_t *out_I, float *out_D, const int32_t *adj,
     a.max_iter = 2 * beam * ef < 1024 ? 2 * beam * ef : 1024;
     a.words_per_slot = p.words_per_slot, a.sort_n = p.sort_n;
     a.slot_stride = p.slot_stride;
-    a.lds_cells = p.lds_cells;
 
     hipStream_t stream = (hipStream_t)stream_;
     reset_work_counter<<<1, 1, 0, stream>>>(a.work_counter);

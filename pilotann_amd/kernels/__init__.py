@@ -242,6 +242,29 @@ def routing_cuda(query: torch.Tensor,
     return router, distances
 
 
+def rotate(query: torch.Tensor, VT: torch.Tensor, n_out: int = None):
+    """``query @ VT.T`` restricted to its first ``n_out`` columns (all of them
+    by default): the rotation of ``IndexStaged.search``
+    (``pilot_ann/layers/staged.py:198-201``) on the device's matrix cores.
+    ``query[B, d]`` and ``VT[d, d]`` are device tensors; returns ``[B, n_out]``
+    on the current stream."""
+    _check(query, 'query', 2, torch.float32, True)
+    _check(VT, 'VT', 2, torch.float32, True)
+    d_model = query.size(-1)
+    _require(VT.size(0) == d_model and VT.size(1) == d_model,
+             'VT.sizes() == {d_model, d_model}')
+    _require(d_model % 8 == 0, 'd_model % 8 == 0')
+    n_out = d_model if n_out is None else int(n_out)
+    _require(1 <= n_out <= d_model, '1 <= n_out <= d_model')
+    out = torch.empty(query.size(0), n_out, dtype=torch.float32,
+                      device=query.device)
+    with torch.cuda.device(query.device):
+        _lib.check(_lib.lib().pa_rotate(
+            _ptr(out), _ptr(query), _ptr(VT), query.size(0), d_model, n_out,
+            _stream()), 'pa_rotate')
+    return out
+
+
 def entry_distances(query: torch.Tensor, entry_vectors: torch.Tensor):
     """Squared L2 from every query to a fixed list of entry vectors
     ``[n_entries, d]`` — what ``IndexEntry.search`` computes with

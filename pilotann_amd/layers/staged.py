@@ -117,6 +117,7 @@ class IndexStaged(nn.Module):
         mapping[sampled] = place[mapping[sampled]]
         self.mapping_cuda = mapping
         if torch.device(device).type == 'cuda':
+            self.VT_cuda = self.VT.to(device)
             kernels.prepare_graph(
                 self.subgraph_cuda.indptr, self.subgraph_cuda.indices,
                 self.mapping_cuda, self.storage_cuda.size(0), self.n_neighbors)
@@ -188,14 +189,25 @@ class IndexStaged(nn.Module):
     # -- search: layers/staged.py:191-228 -------------------------------------
     @torch.no_grad()
     def search(self, query: torch.Tensor, k: int, ef_search: int,
-               chunk_size: int = 128, refine: str = 'host'):
+               chunk_size: int = 128, refine: str = 'host',
+               rotate: str = 'device'):
+        """``rotate='device'`` (default on a GPU) uploads the query and
+        rotates it there (``kernels.rotate``), then copies the rotated query
+        back for the host refine; ``rotate='host'`` is the reference's host
+        matmul (``layers/staged.py:198``).  The two agree to float rounding."""
         assert query.dim() == 2
         if refine == 'device':
             return self._search_on_device(query, k, ef_search)
         assert refine == 'host'
-        query = torch.matmul(query, self.VT.T).contiguous()
-        query_cuda = query[:, :self.d_principle].contiguous().to(
-            device=self.cuda_device)
+        if rotate == 'device' and self.VT_cuda is not None:
+            rotated = kernels.rotate(
+                query.to(device=self.cuda_device).contiguous(), self.VT_cuda)
+            query_cuda = rotated[:, :self.d_principle].contiguous()
+            query = rotated.cpu()
+        else:
+            query = torch.matmul(query, self.VT.T).contiguous()
+            query_cuda = query[:, :self.d_principle].contiguous().to(
+                device=self.cuda_device)
         EP_I, EP_D = self.entry.search(query_cuda)
         return kernels.pipeline(
             graph=[self.fullgraph.indptr, self.fullgraph.indices],
@@ -215,15 +227,13 @@ class IndexStaged(nn.Module):
         searched as two halves on two streams: while the last searches of one
         half's launch finish, the other half's launch fills the idle
         wavefront slots (6 % on the headline configuration; more chunks only
-        add launches).  The rotation runs where ``query`` lives; given the
-        same rotated query the results are those of the host refine."""
+        add launches).  The query is rotated on the device
+        (``kernels.rotate``); given the same rotated query the results are
+        those of the host refine."""
         if self.storage_full_cuda is None:
             self.stage_refine()
         device = self.cuda_device
-        if query.is_cuda:
-            query = torch.matmul(query, self.VT_cuda.T).contiguous()
-        else:
-            query = torch.matmul(query, self.VT.T).contiguous().to(device)
+        query = kernels.rotate(query.to(device).contiguous(), self.VT_cuda)
         query_cuda = query[:, :self.d_principle].contiguous()
         EP_I, EP_D = self.entry.search(query_cuda)
         EP_I, EP_D = EP_I.contiguous(), EP_D.contiguous()

@@ -10,13 +10,14 @@ choice takes a seed.
 """
 from .recall import recall
 from .svd import svd
-from .graphs import knn_graph, graph_init, subgraph_init, graph_sampling
+from .graphs import (knn_graph, graph_init, subgraph_init, graph_sampling,
+                     connect_graph, reachable)
 from .router import router_init
 from .synth import gaussian_mixture, brute_force_topk
 from .layout import locality_order
 
 __all__ = [
     'recall', 'svd', 'knn_graph', 'graph_init', 'subgraph_init',
-    'graph_sampling', 'router_init', 'gaussian_mixture', 'brute_force_topk',
+    'graph_sampling', 'connect_graph', 'reachable', 'router_init', 'gaussian_mixture', 'brute_force_topk',
     'locality_order',
 ]

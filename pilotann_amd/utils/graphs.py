@@ -107,8 +107,104 @@ def _add_reverse(forward: torch.Tensor, degree: int):
     return adj
 
 
+def reachable(adj: torch.Tensor, sources: torch.Tensor, reverse: bool = False):
+    """Boolean mask of the nodes a walk along the edges of ``adj[N, deg]``
+    (``-1`` padded) reaches from ``sources``; with ``reverse`` the nodes from
+    which a walk reaches one of ``sources``."""
+    n = adj.size(0)
+    mark = torch.zeros(n, dtype=torch.bool, device=adj.device)
+    mark[sources] = True
+    if reverse:
+        valid = adj >= 0
+        safe = adj.clamp(min=0)
+        while True:
+            grown = mark | (mark[safe] & valid).any(-1)
+            if bool((grown == mark).all()):
+                return mark
+            mark = grown
+    frontier = sources.flatten()
+    while frontier.numel():
+        nb = adj[frontier].flatten()
+        nb = nb[nb >= 0]
+        frontier = torch.unique(nb[~mark[nb]])
+        mark[frontier] = True
+    return mark
+
+
+def _add_edge(adj, protected, u: int, v: int):
+    """Edge u -> v: into the row's first free slot, else over its farthest
+    neighbour that is not itself an edge added here."""
+    row = adj[u]
+    if u == v or bool((row == v).any()):
+        return
+    free = torch.nonzero(row < 0).flatten()
+    if free.numel():
+        adj[u, int(free[0])] = v
+        return
+    deg = adj.size(1)
+    if int(protected[u]) >= max(1, deg // 4):
+        return
+    adj[u, deg - 1 - int(protected[u])] = v
+    protected[u] += 1
+
+
+def connect_graph(x: torch.Tensor, adj: torch.Tensor, hub: int = None,
+                  max_rounds: int = 32, per_round: int = 1024, seed: int = 0):
+    """Makes every node of ``adj[N, deg]`` reachable from the hub (the node
+    nearest to the mean of ``x``) and the hub reachable from every node, so
+    that a search started anywhere can get everywhere: what faiss' NSG build
+    ensures with its spanning tree from the navigating node and an HNSW base
+    layer gets from incremental insertion, and a pruned k-nearest-neighbour
+    table alone does not (separated clusters stay separate).  Per round, up to
+    ``per_round`` nodes that are cut off are each linked, both ways, with the
+    nearest node that is not; the rest of their cluster follows through its
+    own edges.  Edges go to free slots first, else over the row's farthest
+    neighbours (at most a quarter of a row).  In place; returns the number of
+    rounds used, or -1 if ``max_rounds`` did not suffice."""
+    n, deg = adj.shape
+    dev = adj.device
+    if hub is None:
+        hub = int(torch.argmin((x.float() - x.float().mean(0)).square().sum(-1)))
+    hub_t = torch.tensor([hub], device=dev)
+    protected = torch.zeros(n, dtype=torch.long)
+    g = torch.Generator().manual_seed(seed)
+    xf = x.float()
+    for round_ in range(max_rounds):
+        fwd = reachable(adj, hub_t)
+        bwd = reachable(adj, hub_t, reverse=True)
+        ok = fwd & bwd
+        if bool(ok.all()):
+            return round_
+        cut = torch.nonzero(~ok).flatten()
+        if cut.numel() > per_round:
+            pick = torch.randperm(cut.numel(), generator=g)[:per_round]
+            cut = cut[pick.to(dev)]
+        inside = torch.nonzero(ok).flatten()
+        # connected nodes whose row can still take an edge
+        room = (adj[inside] < 0).any(-1) | \
+            (protected.to(dev)[inside] < max(1, deg // 4))
+        if bool(room.any()):
+            inside = inside[room]
+        # nearest such node of every picked node, in chunks
+        norms = xf[inside].square().sum(-1)
+        nearest = []
+        step = max(1, (1 << 28) // max(1, inside.numel()))
+        for lo in range(0, cut.numel(), step):
+            q = xf[cut[lo:lo + step]]
+            d = norms.unsqueeze(0) - 2.0 * (q @ xf[inside].T)
+            nearest.append(inside[torch.argmin(d, -1)])
+        nearest = torch.cat(nearest)
+        for u, t in zip(cut.tolist(), nearest.tolist()):
+            _add_edge(adj, protected, t, u)
+            _add_edge(adj, protected, u, t)
+    fwd = reachable(adj, hub_t)
+    bwd = reachable(adj, hub_t, reverse=True)
+    return max_rounds if bool((fwd & bwd).all()) else -1
+
+
 def graph_init(x: torch.Tensor, graph_type: str, n_neighbors: int,
-               ef_construct: int = 80, compute_dtype: torch.dtype = None):
+               ef_construct: int = 80, compute_dtype: torch.dtype = None,
+               connect: bool = True):
     """``(indptr, indices)`` int64 tensors on the CPU
     (``pilot_ann/utils/graphs.py:80-93``).
 
@@ -117,7 +213,9 @@ def graph_init(x: torch.Tensor, graph_type: str, n_neighbors: int,
     M = n_neighbors/2 (``graphs.py:52-54``).  ``nsg``: up to ``n_neighbors``
     pruned forward edges without filling, then reverse edges where room is
     left, so rows can end in ``-1`` padding as faiss' NSG rows do.
-    ``ef_construct`` bounds the candidate pool per node."""
+    ``ef_construct`` bounds the candidate pool per node.  With ``connect``
+    (default) :func:`connect_graph` then links what the neighbour table left
+    cut off."""
     if x.dim() != 2:
         raise RuntimeError
     n = x.size(0)
@@ -132,18 +230,24 @@ def graph_init(x: torch.Tensor, graph_type: str, n_neighbors: int,
     else:
         raise RuntimeError
     adj = _add_reverse(fwd, n_neighbors)
+    if connect and n > 1:
+        connect_graph(x, adj)
     indptr = torch.arange(n + 1, dtype=torch.long) * n_neighbors
     return indptr, adj.flatten().cpu()
 
 
 def graph_sampling(indptr: torch.Tensor, indices: torch.Tensor,
                    n_samples: int, n_hops: int, seed: int = 0,
-                   device: str = 'cpu'):
-    """Seeded version of ``extension/sampling_cpu.cpp:5-65``: random seed
-    nodes, each with its ``n_hops`` neighbourhood, are added in a fixed random
-    order until at least ``n_samples`` nodes are in.  Returns the sorted
-    ``nodelist`` and ``mapping`` (global id → position in nodelist, else -1).
-    """
+                   device: str = 'cpu', return_seeds: bool = False):
+    """Seeded version of ``extension/sampling_cpu.cpp:5-65``.  The reference
+    draws seed nodes one after the other and adds each with everything within
+    ``n_hops`` edges of it, until at least ``n_samples`` nodes are in; the
+    same here, with the seeds taken from a seeded random order of the nodes
+    (the reference seeds ``rand()`` with the time).  As the sample only grows
+    with every seed, the stopping point is found by bisection over the number
+    of seeds instead of one seed at a time.  Returns the sorted ``nodelist``
+    and ``mapping`` (global id → position in nodelist, else -1), and the
+    seeds used with ``return_seeds``."""
     indptr = torch.as_tensor(indptr, dtype=torch.long).to(device)
     indices = torch.as_tensor(indices, dtype=torch.long).to(device)
     n = indptr.numel() - 1
@@ -170,6 +274,8 @@ def graph_sampling(indptr: torch.Tensor, indices: torch.Tensor,
     nodelist = torch.nonzero(closure(lo)).flatten().cpu()
     mapping = torch.full((n,), -1, dtype=torch.long)
     mapping[nodelist] = torch.arange(nodelist.numel())
+    if return_seeds:
+        return nodelist, mapping, order[:lo].cpu()
     return nodelist, mapping
 
 

@@ -44,6 +44,10 @@ def test_host_only_entry_points():
                                4, 100, 60, 8, 10, 16) == -3
     assert lib.pa_pipeline(*([None] * 15), 100, 1000, 250, 64, 32, 32, 32, 16,
                            10, 30, None) == -9
+    assert lib.pa_rotate(None, None, None, 4, 60, 8, None) == -3
+    assert lib.pa_rotate(None, None, None, 4, 64, 65, None) == -2
+    assert lib.pa_rotate(None, None, None, 4, 64, 8, None) == -1
+    assert lib.pa_rotate(None, None, None, 0, 64, 8, None) == 0
     # pa_graph_prepare: sizes first (indices of a negative length), then the
     # pointers; the content of indptr is checked on the device
     assert lib.pa_graph_prepare(None, None, None, 100, 50, -1, 32, None, None,

@@ -98,7 +98,7 @@ def test_index_staged_end_to_end(device):
     again_I, again_D = index.search(q, k=k, ef_search=32, chunk_size=512)
     assert torch.equal(again_I, top_I) and torch.equal(again_D, top_D)
     # the refine on the device gives the host refine's answer (same rotated
-    # query: a host query is rotated on the host in both)
+    # query: both rotate it on the device)
     dev_I, dev_D = index.search(q, k=k, ef_search=32, refine='device')
     assert not dev_I.is_cuda
     assert_same_search(dev_I.numpy(), dev_D.numpy(), top_I.numpy(), top_D.numpy())
@@ -107,9 +107,15 @@ def test_index_staged_end_to_end(device):
     for i in range(5):
         assert torch.equal(big_I[512 * i:512 * (i + 1)], dev_I)
         assert torch.equal(big_D[512 * i:512 * (i + 1)], dev_D)
-    # a device query is rotated there: another matrix product, same quality
+    # a query that is already on the device: same rotation, same answer
     gpu_I, gpu_D = index.search(q.to(device), k=k, ef_search=32, refine='device')
-    assert abs(utils.recall(gpu_I, target) - utils.recall(top_I, target)) < 0.005
+    assert torch.equal(gpu_I, dev_I) and torch.equal(gpu_D, dev_D)
+    # the reference's host matmul instead: another summation order, results
+    # of the same quality
+    host_I, host_D = index.search(q, k=k, ef_search=32, chunk_size=128,
+                                  rotate='host')
+    assert abs(utils.recall(host_I, target) - utils.recall(top_I, target)) < 0.005
+    assert float((host_I == top_I).float().mean()) > 0.99
     # a reloaded checkpoint searches identically
     import io
     blob = io.BytesIO()

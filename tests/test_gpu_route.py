@@ -96,3 +96,33 @@ def test_routing_random_shapes(seed, device):
         oracle.square_dist(q[b].numpy(), flat, entry_nodes[router[b]].numpy().copy())
         for b in range(B)])
     assert np.array_equal(dist, ref)
+
+
+@pytest.mark.parametrize('B,d,n_out', [
+    (1, 8, 8), (31, 64, 32), (64, 96, 64), (100, 200, 40), (1000, 768, 128),
+    (257, 768, 768), (65, 72, 1),
+])
+def test_rotation_matches_float64_matmul(B, d, n_out, device):
+    """`pa_rotate` (query @ VT.T, first n_out columns) against a float64
+    product of the same float32 inputs.  Tolerance: float32 accumulation of d
+    products, |error| <= 4 d eps |q| |v| (eps = 2^-24), far inside the 1e-5
+    relative the search's distances are held to."""
+    print('rotate case', B, d, n_out, flush=True)
+    g = torch.Generator().manual_seed(B + d)
+    query = torch.randn(B, d, generator=g)
+    basis, _ = torch.linalg.qr(torch.randn(d, d, generator=g))
+    VT = basis.T.contiguous()
+    out = kernels.rotate(query.to(device), VT.to(device), n_out)
+    torch.cuda.synchronize()
+    assert out.shape == (B, n_out)
+    ref = (query.double() @ VT.double().T)[:, :n_out]
+    bound = 4 * d * 2.0 ** -24 * query.double().norm(dim=1, keepdim=True) \
+        * VT.double().norm(dim=1)[:n_out].unsqueeze(0)
+    assert bool(((out.cpu().double() - ref).abs() <= bound).all())
+    # the rotation preserves lengths when all columns are kept
+    if n_out == d:
+        assert torch.allclose(out.cpu().norm(dim=1), query.norm(dim=1), rtol=1e-5)
+    with pytest.raises(RuntimeError):
+        kernels.rotate(query.to(device), VT.to(device), d + 1)
+    with pytest.raises(RuntimeError):
+        kernels.rotate(query, VT.to(device))

@@ -112,3 +112,77 @@ def test_locality_order_is_a_permutation_that_groups_neighbours():
     old_gap = (x[1:] - x[:-1]).norm(dim=1).mean()
     assert new_gap < 0.5 * old_gap
     assert utils.locality_order(x[:5]).numel() == 5
+
+
+def test_sampling_follows_the_reference_rule_on_a_hand_built_graph():
+    """extension/sampling_cpu.cpp:38-47: seeds are added, each with all nodes
+    within n_hops edges, until the sample has n_samples nodes.  Graph: six
+    stars 4k -> {4k+1, 4k+2, 4k+3} whose leaves have no edges, leaves of star
+    k also point at the centre of star k+1 through node 4k+3."""
+    n = 24
+    rows = [[] for _ in range(n)]
+    for k in range(6):
+        rows[4 * k] = [4 * k + 1, 4 * k + 2, 4 * k + 3]
+        rows[4 * k + 3] = [4 * ((k + 1) % 6)]
+    indptr = torch.tensor([0] + [len(r) for r in rows]).cumsum(0)
+    indices = torch.tensor([v for r in rows for v in r])
+
+    def closure(seeds, hops):
+        got = set(seeds)
+        for s in seeds:
+            frontier = {s}
+            for _ in range(hops):
+                frontier |= {v for u in frontier for v in rows[u]}
+            got |= frontier
+        return got
+
+    for hops, want in ((1, 9), (2, 9), (1, 24)):
+        for seed in range(5):
+            nodelist, mapping, seeds = utils.graph_sampling(
+                indptr, indices, want, hops, seed=seed, return_seeds=True)
+            seeds = seeds.tolist()
+            assert set(nodelist.tolist()) == closure(seeds, hops)
+            assert len(nodelist) >= want
+            # the last seed was needed: without it the sample is too small
+            assert len(closure(seeds[:-1], hops)) < want
+            assert (mapping[nodelist] == torch.arange(len(nodelist))).all()
+            assert int((mapping >= 0).sum()) == len(nodelist)
+
+
+def test_connectivity_pass_joins_separated_clusters():
+    """Well separated clusters: the neighbour table alone leaves one island
+    per cluster; after the pass every node is reachable from every node, the
+    row format is intact and the searches of the reference's own graph test
+    (test/kernel/test_graphs.py:55-64) find their neighbours from entries in
+    another cluster."""
+    n, d, deg = 4000, 32, 16
+    x = utils.gaussian_mixture(n, d, 16, 0.05, seed=8)
+    for graph_type in ['nsw', 'nsg']:
+        _, loose = utils.graph_init(x, graph_type, deg, connect=False)
+        loose = loose.view(n, deg)
+        assert not bool(utils.reachable(loose, torch.tensor([0])).all())
+        indptr, indices = utils.graph_init(x, graph_type, deg)
+        rows = indices.view(n, deg)
+        for start in (0, 1234, n - 1):
+            assert bool(utils.reachable(rows, torch.tensor([start])).all())
+            assert bool(utils.reachable(rows, torch.tensor([start]), reverse=True).all())
+        valid = rows >= 0
+        assert (valid[:, :-1] | ~valid[:, 1:]).all()
+        assert not (rows == torch.arange(n).unsqueeze(1)).any()
+        srt = torch.sort(torch.where(valid, rows, -torch.arange(1, deg + 1)), 1).values
+        assert (srt[:, 1:] != srt[:, :-1]).all()
+        # a search from one fixed entry reaches the neighbours of queries of
+        # every cluster
+        import numpy as np
+        import oracle
+        q = utils.gaussian_mixture(64, d, 16, 0.05, seed=9, center_seed=8)
+        target = utils.brute_force_topk(q, x, 10)
+        init_I = torch.zeros(64, 1, dtype=torch.long)
+        init_D = (q - x[0]).square().sum(-1, keepdim=True)
+        out_I = np.empty((64, 10), np.int64)
+        out_D = np.empty((64, 10), np.float32)
+        oracle.traverse_cpu(out_I, out_D, init_I.numpy(), init_D.numpy().copy(),
+                            indptr.numpy(), indices.numpy(), x.numpy(), q.numpy(), 64)
+        # (0.08 on the table without the pass: one cluster of sixteen; the
+        # bridges are few, so a greedy search does not always find them)
+        assert utils.recall(torch.from_numpy(out_I), target) > 0.5
