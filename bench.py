@@ -387,39 +387,28 @@ def cpu_baseline(index, stage, ef, EP_I, EP_D, budget_s=8.0):
     return base, results['plain_c_port']
 
 
-def cpu_full_graph_baseline(index, stage, EP_I, target, k, budget_s=6.0):
-    """The search without a GPU: the host search on the full graph in full
-    dimension from the same entry ids (their full-dimension distances are
-    computed on the host, inside the timed region), at the smallest ef_search
-    whose recall@k reaches 0.90 on a 2000-query sample — the role faiss' HNSW
-    plays in the reference's own table (README.md:527-534)."""
+def cpu_full_graph_baseline(index, query, stage, target, k, budget_s=6.0):
+    """The search without a GPU (`IndexStaged.search_cpu`: rotation, the
+    router's entries with full-dimension distances and the host search on the
+    full graph in full dimension, all inside the timed region), at the
+    smallest ef_search whose recall@k reaches 0.90 on a 2000-query sample —
+    the role faiss' HNSW plays in the reference's own table
+    (README.md:527-534)."""
     import oracle
-    from pilotann_amd import kernels, utils
+    from pilotann_amd import utils
     if index.fullgraph is None:
         return None
-    indptr, indices = index.fullgraph.indptr, index.fullgraph.indices
-    storage, query = index.storage, stage.query_rot
-    ids = EP_I.cpu()
 
-    def run(lo, hi, ef_search):
-        q = query[lo:hi].contiguous()
+    def run(n, ef_search):
         t0 = time.perf_counter()
-        i = ids[lo:hi].contiguous()
-        d = torch.empty(i.shape, dtype=torch.float)
-        for a in range(0, hi - lo, 500):
-            rows = storage[i[a:a + 500]]
-            d[a:a + 500] = (q[a:a + 500].unsqueeze(1) - rows).square().sum(-1)
-        out_I = torch.empty(hi - lo, k, dtype=torch.long)
-        out_D = torch.empty(hi - lo, k, dtype=torch.float)
-        kernels.traverse_cpu(out_I, out_D, i, d, indptr, indices, storage, q,
-                             ef_search)
+        out_I, _ = index.search_cpu(query[:n], k=k, ef_search=ef_search)
         return time.perf_counter() - t0, out_I
 
     n_sample = min(2000, stage.B)
     sweep, chosen = [], None
     for ef_search in [e for e in (16, 24, 32, 48, 64, 96, 128, 192, 256, 384,
                                   512, 1024) if e >= k]:
-        t, out_I = run(0, n_sample, ef_search)
+        t, out_I = run(n_sample, ef_search)
         rec = utils.recall(out_I, target[:n_sample])
         sweep.append(dict(ef_search=ef_search, recall=round(rec, 4)))
         if rec >= 0.90:
@@ -429,13 +418,14 @@ def cpu_full_graph_baseline(index, stage, EP_I, target, k, budget_s=6.0):
         chosen = sweep[-1]['ef_search']
     total_t, total_n, passes, rec = 0.0, 0, 0, None
     while total_t < budget_s and passes < 100:
-        t, out_I = run(0, stage.B, chosen)
+        t, out_I = run(stage.B, chosen)
         rec = utils.recall(out_I, target)
         total_t += t
         total_n += stage.B
         passes += 1
-    return dict(what='traverse_cpu (library host search, AVX2) on the full '
-                     'graph in full dimension, entry distances included',
+    return dict(what='IndexStaged.search_cpu: rotation, router entries and '
+                     'traverse_cpu (library host search, AVX2) on the full '
+                     'graph in full dimension',
                 ef_search=chosen, recall_at_k=round(rec, 4),
                 queries_per_s=round(total_n / total_t, 1),
                 cores=oracle.num_threads(), passes=passes, sweep=sweep)
@@ -611,7 +601,7 @@ def main():
         line['config']['matches_cpu_baseline'] = compare_search(
             out_I.flatten(1).cpu().numpy(), out_D.flatten(1).cpu().numpy(),
             ref_I, ref_D)
-        full = cpu_full_graph_baseline(index, stage, EP_I, target, k)
+        full = cpu_full_graph_baseline(index, query, stage, target, k)
         if full:
             line['cpu_baseline']['without_gpu'] = full
     print(json.dumps(line), flush=True)

@@ -137,8 +137,12 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
         PA_TIMER_BEGIN();
 
         // fresh visited slice, query to LDS, empty lists
-        for (int w = lane * 4; w < a.words_per_slot; w += kWave * 4)
-            *reinterpret_cast<uint4 *>(seen + w) = make_uint4(0, 0, 0, 0);
+#ifndef PA_CLEAR_REPS  // tuning builds: the clearing repeated, to time it
+#define PA_CLEAR_REPS 1
+#endif
+        for (int rep = 0; rep < PA_CLEAR_REPS; ++rep)
+            for (int w = lane * 4; w < a.words_per_slot; w += kWave * 4)
+                *reinterpret_cast<uint4 *>(seen + w) = make_uint4(0, 0, 0, 0);
         for (int i = lane; i < dp; i += kWave)
             qv[query_slot(i, dp >> 3)] = a.query[(size_t)q * dp + i];
         for (int i = lane; i < kSeenCache; i += kWave) seen_cache[i] = 0xffffffffu;

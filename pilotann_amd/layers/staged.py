@@ -221,6 +221,37 @@ class IndexStaged(nn.Module):
             ef_search=ef_search, d_principle=self.d_principle,
             chunk_size=chunk_size)
 
+    @torch.no_grad()
+    def search_cpu(self, query: torch.Tensor, k: int, ef_search: int):
+        """The search without a device, as a baseline: rotation on the host,
+        the entry ids the router would give (nearest route vector over the
+        first ``d_principle`` coordinates) with their full-dimension
+        distances, then ``traverse_cpu`` on the full graph in full dimension.
+        Not part of the reference's index; it plays the role faiss' HNSW has
+        in the reference's benchmark (``script/common.py:103-120``)."""
+        query = torch.matmul(query.cpu(), self.VT.T).contiguous()
+        entry = self.entry
+        nodes = entry.entry_nodes.cpu()
+        batch = query.size(0)
+        if entry.route_vectors is not None:
+            route = torch.cdist(query[:, :self.d_principle],
+                                entry.route_vectors.cpu()).argmin(-1)
+            ids = nodes[route].contiguous()
+            dist = torch.empty(ids.shape, dtype=torch.float)
+            for r in torch.unique(route).tolist():
+                rows = torch.nonzero(route == r).flatten()
+                leaves = self.storage[nodes[r]]
+                dist[rows] = torch.cdist(query[rows], leaves).square()
+        else:
+            ids = nodes.unsqueeze(0).expand(batch, -1).contiguous()
+            dist = torch.cdist(query, self.storage[nodes]).square().contiguous()
+        topk_I = torch.empty(batch, k, dtype=torch.long)
+        topk_D = torch.empty(batch, k, dtype=torch.float)
+        kernels.traverse_cpu(topk_I, topk_D, ids, dist, self.fullgraph.indptr,
+                             self.fullgraph.indices, self.storage, query,
+                             max(ef_search, k))
+        return topk_I, topk_D
+
     def _search_on_device(self, query, k, ef_search):
         """All three stages on the device: entries, subgraph traversal, refine,
         top-k copied back at the end.  A batch of 2048 queries or more is

@@ -125,3 +125,23 @@ def test_index_staged_end_to_end(device):
     clone.to(device)
     clone_I, clone_D = clone.search(q, k=k, ef_search=32, chunk_size=128)
     assert torch.equal(clone_I, top_I) and torch.equal(clone_D, top_D)
+
+
+def test_command_line_benchmark_prints_the_reference_lines(device, capsys):
+    """script/bench_1.py:57-60: one `method: recall=…, duration=…ms` line per
+    ef_search and method, then the records."""
+    import re
+    from pilotann_amd import cli
+    records = cli.main(['--dataset', 'synth:20000x64:16:0.5', '--d_principle', '32',
+                        '--n_neighbors', '32', '--router', 'router16x32',
+                        '--ef_search', '16,32', '--n_queries', '256',
+                        '--n_repeats', '3', '--device', str(device)])
+    out = capsys.readouterr().out
+    lines = re.findall(r'^(search-pilot|host-cpu): recall=(\d\.\d{3}), '
+                       r'duration=(\d+\.\d{3})ms$', out, flags=re.M)
+    assert [m for m, _, _ in lines] == ['search-pilot'] * 2 + ['host-cpu'] * 2
+    assert all(0.5 < float(r) <= 1.0 for _, r, _ in lines)
+    assert set(records) == {'search-pilot', 'host-cpu'}
+    assert [r['ef_search'] for r in records['search-pilot']] == [16, 32]
+    # more effort, better recall
+    assert records['search-pilot'][1]['recall'] >= records['search-pilot'][0]['recall']

@@ -54,3 +54,19 @@ def test_index_staged_train_dump_load():
         b = clone.state_dict()[name]
         assert torch.equal(a, b), name
     assert clone.n_neighbors == 16 and clone.d_principle == 16
+
+
+def test_search_cpu_is_the_whole_search_on_the_host():
+    """`IndexStaged.search_cpu`: rotation, router entries, host search on the
+    full graph — finds the true neighbours and reports full-dimension
+    distances (a rotation keeps them)."""
+    x = utils.gaussian_mixture(6000, 64, 16, 1.0, seed=1, decay=0.5)
+    q = utils.gaussian_mixture(100, 64, 16, 1.0, seed=2, center_seed=1, decay=0.5)
+    target = utils.brute_force_topk(q, x, 10)
+    for entry_method in ('router8x32', 'random32'):
+        index = layers.IndexStaged(64, 32, 0.25, 'nsw32', entry_method, seed=3)
+        index.train(x)
+        top_I, top_D = index.search_cpu(q, 10, 64)
+        assert utils.recall(top_I, target) > 0.95
+        ref = (q.unsqueeze(1) - x[top_I]).square().sum(-1)
+        assert torch.allclose(top_D, ref, atol=1e-3)
