@@ -46,7 +46,8 @@ CONFIGS = {
     'c3': dict(n=1_000_000, d=768, dp=128, n_centers=1024, sigma=1.0,
                decay=0.5, normalize=True, ratio=0.25, graph='nsw64',
                entry='router64x64', queries=10_000, k=10,
-               ef_sweep=[4, 8, 16, 24, 32, 48, 64], seed=301),
+               ef_sweep=[4, 8, 16, 24, 32, 48, 64], seed=301,
+               curve=[32, 48, 64, 96, 128, 192, 256]),
     # large result lists: top-100, ef 256 / 512 (heaps of 1024 / 2048 entries)
     'c4': dict(n=1_000_000, d=768, dp=128, n_centers=1024, sigma=1.0,
                decay=0.5, normalize=True, ratio=0.5, graph='nsw64',
@@ -167,8 +168,10 @@ class Stage:
         self.kernels = kernels
         self.index = index
         self.device = device
-        self.query_rot = torch.matmul(query, index.VT.T).contiguous()
-        self.query_cuda = self.query_rot[:, :index.d_principle].contiguous().to(device)
+        # rotated on the device, as IndexStaged.search does (kernels.rotate)
+        rotated = kernels.rotate(query.to(device).contiguous(), index.VT_cuda)
+        self.query_rot = rotated.cpu()
+        self.query_cuda = rotated[:, :index.d_principle].contiguous()
         self.graph = kernels.prepare_graph(
             index.subgraph_cuda.indptr, index.subgraph_cuda.indices,
             index.mapping_cuda, index.storage_cuda.size(0), index.n_neighbors)
@@ -524,7 +527,10 @@ def main():
     # pick ef: smallest of the sweep with end-to-end recall@k >= 0.90
     sweep = []
     chosen = None
-    for ef in ([args.ef] if args.ef else cfg['ef_sweep']):
+    efs = [args.ef] if args.ef else cfg['ef_sweep']
+    if args.curve and not args.ef:
+        efs = cfg.get('curve', efs)
+    for ef in efs:
         rec, refine_s = end_to_end_recall(index, stage, ef, target, k)
         sweep.append(dict(ef=ef, recall=round(rec, 4),
                           refine_qps=round(B / refine_s, 1)
@@ -571,7 +577,7 @@ def main():
         },
         'roofline': stage_record(t, B, key),
     }
-    others = [e for e in (cfg['ef_sweep'] if args.curve else
+    others = [e for e in (efs if args.curve else
                           ALSO_TIMED.get(args.config, []))
               if e != ef and not args.ef]
     if others:

@@ -58,6 +58,7 @@ class IndexStaged(nn.Module):
         self.fullgraph_cuda = None
         self.storage_full_cuda = None
         self.VT_cuda = None
+        self._full_prepared = None
         self._streams = None
 
     # -- checkpoint: layers/staged.py:59-122 ---------------------------------
@@ -149,8 +150,10 @@ class IndexStaged(nn.Module):
         self.VT_cuda = self.VT.to(device)
         self.fullgraph_cuda = GraphModule(self.fullgraph.indptr,
                                           self.fullgraph.indices).to(device)
-        kernels.prepare_full_graph(self.fullgraph_cuda.indptr,
-                                   self.fullgraph_cuda.indices)
+        # kept: a later search neither measures the longest row again (a
+        # reduction and a device synchronisation) nor looks the graph up
+        self._full_prepared = kernels.prepare_full_graph(
+            self.fullgraph_cuda.indptr, self.fullgraph_cuda.indices)
         return self
 
     # -- build: layers/staged.py:141-189 --------------------------------------
@@ -278,8 +281,7 @@ class IndexStaged(nn.Module):
         sub = kernels.prepare_graph(
             self.subgraph_cuda.indptr, self.subgraph_cuda.indices,
             self.mapping_cuda, self.storage_cuda.size(0), self.n_neighbors)
-        full = kernels.prepare_full_graph(self.fullgraph_cuda.indptr,
-                                          self.fullgraph_cuda.indices)
+        full = self._full_prepared
 
         def run(lo, hi):
             kernels.traverse_prepared(
