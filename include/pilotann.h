@@ -175,13 +175,18 @@ int pa_traverse_static(int64_t *out_I, float *out_D, const int32_t *adj,
  *          leaf vector of its route, entry_vectors[router[b], l, :].
  *   query [batch * dp], route_vectors [n_routers * dp],
  *   entry_vectors [n_routers * n_leaves * dp], all float.
+ *   entry_nodes [n_routers * n_leaves] int64 and entry_ids [batch * n_leaves]
+ *          int64, out: both NULL, or the ids of the chosen route's leaves are
+ *          written as well, entry_ids[b][l] = entry_nodes[router[b]][l] — the
+ *          `index_select` that follows the call in pilot_ann/layers/entry.py:86.
  * With n_routers == 0 every query uses group 0 of entry_vectors and `router`
  * may be NULL: the distances of a fixed entry list
  * (pilot_ann/layers/entry.py:70-77).
  */
 int pa_route(int64_t *router, float *dist, const float *query,
              const float *route_vectors, const float *entry_vectors,
-             int64_t batch, int n_routers, int n_leaves, int dp, void *stream);
+             int64_t batch, int n_routers, int n_leaves, int dp,
+             const int64_t *entry_nodes, int64_t *entry_ids, void *stream);
 
 /*
  * Replaces the query rotation of `IndexStaged.search`

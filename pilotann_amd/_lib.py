@@ -28,7 +28,7 @@ _SIGNATURES = {
                                   _i64, _i64, _i64, _int, _int, _int, _int,
                                   _int, _vp, _vp]),
     'pa_route': (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _int,
-                        _vp]),
+                        _vp, _vp, _vp]),
     'pa_rotate': (_int, [_vp, _vp, _vp, _i64, _int, _int, _vp]),
     'pa_traverse_cpu': (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                                _i64, _i64, _int, _int, _int, _int]),

@@ -52,9 +52,11 @@ __global__ __launch_bounds__(kWave) void route_score_kernel(
         const bool r_ok = rj < n_routers;
         const float4 *rrow =
             reinterpret_cast<const float4 *>(routes + (size_t)(r_ok ? rj : 0) * dp) + half;
-        floatx16 acc;
+        // two accumulators take alternate instructions: none waits for the
+        // result of the one before it
+        floatx16 acc, acc_odd;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+        for (int r = 0; r < 16; ++r) acc[r] = 0.f, acc_odd[r] = 0.f;
         float norm = 0.f;
         for (int c = 0; c < groups; ++c) {
             float4 a = qrow[2 * c];
@@ -66,10 +68,12 @@ __global__ __launch_bounds__(kWave) void route_score_kernel(
             norm = fmaf(b.z, b.z, norm);
             norm = fmaf(b.w, b.w, norm);
             acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b.x, acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b.y, acc, 0, 0, 0);
+            acc_odd = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b.y, acc_odd, 0, 0, 0);
             acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, b.z, acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, b.w, acc, 0, 0, 0);
+            acc_odd = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, b.w, acc_odd, 0, 0, 0);
         }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[r] += acc_odd[r];
         norm += __shfl_xor(norm, 32);
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
@@ -99,8 +103,9 @@ __global__ __launch_bounds__(kWave) void route_score_kernel(
 template <int DP8>
 __global__ __launch_bounds__(256) void leaf_dist_kernel(
     const float *__restrict__ query, const float *__restrict__ entry_vectors,
-    const int64_t *__restrict__ router, float *__restrict__ dist, int batch,
-    int n_leaves, int dp) {
+    const int64_t *__restrict__ router, float *__restrict__ dist,
+    const int64_t *__restrict__ entry_nodes, int64_t *__restrict__ entry_ids,
+    int batch, int n_leaves, int dp) {
     extern __shared__ __align__(16) float qv_all[];
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave;
@@ -113,6 +118,11 @@ __global__ __launch_bounds__(256) void leaf_dist_kernel(
     if (q >= batch) return;
     const int64_t group = router ? router[q] : 0;
     const float *leaves = entry_vectors + (size_t)group * n_leaves * dp;
+    // layers/entry.py:86: the ids of the chosen group's leaves
+    if (entry_ids)
+        for (int l = lane; l < n_leaves; l += kWave)
+            entry_ids[(size_t)q * n_leaves + l] =
+                entry_nodes[(size_t)group * n_leaves + l];
     const int quad = lane >> 2, part = lane & 3;
     const float2 *qq = reinterpret_cast<const float2 *>(qv) + part * query_run(dp >> 3);
     for (int base = 0; base < n_leaves; base += kRowsPerPass) {
@@ -130,6 +140,7 @@ __global__ __launch_bounds__(256) void leaf_dist_kernel(
 extern "C" int pa_route(int64_t *router, float *dist, const float *query,
                         const float *route_vectors, const float *entry_vectors,
                         int64_t batch, int n_routers, int n_leaves, int dp,
+                        const int64_t *entry_nodes, int64_t *entry_ids,
                         void *stream_) {
     if (batch < 0 || n_routers < 0 || n_leaves < 1) return PA_E_SHAPE;
     if (batch >= (1ll << 31)) return PA_E_RANGE;
@@ -138,6 +149,7 @@ extern "C" int pa_route(int64_t *router, float *dist, const float *query,
     if (batch == 0) return PA_OK;
     if (!dist || !query || !entry_vectors) return PA_E_NULL;
     if (n_routers > 0 && (!router || !route_vectors)) return PA_E_NULL;
+    if (entry_ids && !entry_nodes) return PA_E_NULL;
     hipStream_t stream = (hipStream_t)stream_;
     if (n_routers > 0) {
         const unsigned blocks = (unsigned)((batch + kTile - 1) / kTile);
@@ -151,19 +163,23 @@ extern "C" int pa_route(int64_t *router, float *dist, const float *query,
     switch (dp) {
         case 32:
             leaf_dist_kernel<4><<<blocks, waves * kWave, lds, stream>>>(
-                query, entry_vectors, group, dist, (int)batch, n_leaves, dp);
+                query, entry_vectors, group, dist, entry_nodes, entry_ids, (int)batch,
+                n_leaves, dp);
             break;
         case 64:
             leaf_dist_kernel<8><<<blocks, waves * kWave, lds, stream>>>(
-                query, entry_vectors, group, dist, (int)batch, n_leaves, dp);
+                query, entry_vectors, group, dist, entry_nodes, entry_ids, (int)batch,
+                n_leaves, dp);
             break;
         case 128:
             leaf_dist_kernel<16><<<blocks, waves * kWave, lds, stream>>>(
-                query, entry_vectors, group, dist, (int)batch, n_leaves, dp);
+                query, entry_vectors, group, dist, entry_nodes, entry_ids, (int)batch,
+                n_leaves, dp);
             break;
         default:
             leaf_dist_kernel<0><<<blocks, waves * kWave, lds, stream>>>(
-                query, entry_vectors, group, dist, (int)batch, n_leaves, dp);
+                query, entry_vectors, group, dist, entry_nodes, entry_ids, (int)batch,
+                n_leaves, dp);
     }
     return (int)hipGetLastError();
 }

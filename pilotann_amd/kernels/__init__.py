@@ -209,10 +209,14 @@ def traverse_prepared(output_I, output_D, graph: PreparedGraph, storage,
 def routing_cuda(query: torch.Tensor,
                  route_vectors: torch.Tensor,
                  entry_nodes: torch.Tensor,
-                 entry_vectors: torch.Tensor):
+                 entry_vectors: torch.Tensor,
+                 return_entries: bool = False):
     """``kernels.routing_cuda`` (``pilot_ann/kernels/__init__.py:97-103``,
     checks of ``routing_cuda.cu:76-90``): returns ``(router[B] int64,
-    distances[B, n_leaves] float32)``."""
+    distances[B, n_leaves] float32)``.  With ``return_entries`` the ids of the
+    chosen route's leaves, ``entry_nodes[router]`` ``[B, n_leaves]``, are
+    written by the same launch and returned as a third tensor (the
+    ``index_select`` of ``layers/entry.py:86``)."""
     _check(query, 'query', 2, torch.float32, True)
     _check(route_vectors, 'route_vectors', 2, torch.float32, True)
     _check(entry_vectors, 'entry_vectors', 3, torch.float32, True)
@@ -231,14 +235,23 @@ def routing_cuda(query: torch.Tensor,
              'entry_vectors.size(1) == n_leaves')
     _require(n_leaves % 32 == 0, 'n_leaves % BLOCK_SIZE == 0')
     _require(d_model % 8 == 0, 'd_model % 8 == 0')
+    _require(entry_nodes.size(0) == n_routers,
+             'entry_nodes.size(0) == n_routers')
     router = torch.empty(batch_size, dtype=torch.int64, device=query.device)
     distances = torch.empty(batch_size, n_leaves, dtype=torch.float32,
                             device=query.device)
+    entries = None
+    if return_entries:
+        entries = torch.empty(batch_size, n_leaves, dtype=torch.int64,
+                              device=query.device)
     with torch.cuda.device(query.device):
         _lib.check(_lib.lib().pa_route(
             _ptr(router), _ptr(distances), _ptr(query), _ptr(route_vectors),
             _ptr(entry_vectors), batch_size, n_routers, n_leaves, d_model,
+            _ptr(entry_nodes) if return_entries else None, _ptr(entries),
             _stream()), 'pa_route')
+    if return_entries:
+        return router, distances, entries
     return router, distances
 
 
@@ -280,8 +293,8 @@ def entry_distances(query: torch.Tensor, entry_vectors: torch.Tensor):
     with torch.cuda.device(query.device):
         _lib.check(_lib.lib().pa_route(
             None, _ptr(distances), _ptr(query), None, _ptr(entry_vectors),
-            query.size(0), 0, entry_vectors.size(0), query.size(-1),
-            _stream()), 'pa_route')
+            query.size(0), 0, entry_vectors.size(0), query.size(-1), None,
+            None, _stream()), 'pa_route')
     return distances
 
 

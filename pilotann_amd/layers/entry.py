@@ -76,8 +76,7 @@ class IndexEntry(nn.Module):
         else:
             assert query.is_cuda is True
             assert self.entry_vectors.dim() == 3
-            router, EP_D = kernels.routing_cuda(
+            _, EP_D, EP_I = kernels.routing_cuda(
                 query, self.route_vectors, entry_nodes=self.entry_nodes,
-                entry_vectors=self.entry_vectors)
-            EP_I = torch.index_select(self.entry_nodes, dim=0, index=router)
+                entry_vectors=self.entry_vectors, return_entries=True)
         return EP_I, EP_D

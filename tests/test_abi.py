@@ -37,9 +37,9 @@ def test_host_only_entry_points():
     assert lib.pa_error_string(0) == b'ok'
     assert b'multiple of 8' in lib.pa_error_string(-3)
     # argument errors are detected on the host, before any device call
-    assert lib.pa_route(None, None, None, None, None, 4, 8, 24, 64, None) == -8
-    assert lib.pa_route(None, None, None, None, None, 4, 8, 32, 60, None) == -3
-    assert lib.pa_route(None, None, None, None, None, 4, 8, 32, 64, None) == -1
+    assert lib.pa_route(None, None, None, None, None, 4, 8, 24, 64, None, None, None) == -8
+    assert lib.pa_route(None, None, None, None, None, 4, 8, 32, 60, None, None, None) == -3
+    assert lib.pa_route(None, None, None, None, None, 4, 8, 32, 64, None, None, None) == -1
     assert lib.pa_traverse_cpu(None, None, None, None, None, None, None, None,
                                4, 100, 60, 8, 10, 16) == -3
     assert lib.pa_pipeline(*([None] * 15), 100, 1000, 250, 64, 32, 32, 32, 16,

@@ -39,6 +39,13 @@ def test_routing_matches_oracle(R, L, d, B, device):
     # the reference's own check (test_routing.py:69-85)
     target = torch.cdist(q.unsqueeze(1), x[entry_nodes[router]]).square()
     assert torch.allclose(torch.from_numpy(dist), target.squeeze(1), atol=1e-3)
+    # the same launch can hand back the chosen route's entry ids
+    r2, d2, ids = kernels.routing_cuda(
+        q.to(device), route_vectors.contiguous().to(device),
+        entry_nodes.to(device), entry_vectors.to(device), return_entries=True)
+    assert np.array_equal(r2.cpu().numpy(), router)
+    assert np.array_equal(d2.cpu().numpy(), dist)
+    assert torch.equal(ids.cpu(), entry_nodes[torch.from_numpy(router)])
 
 
 def test_entry_distances(device):
