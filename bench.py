@@ -20,7 +20,6 @@ and on the device, are the top-level fields `end_to_end_qps_host_refine` and
 """
 import argparse
 import contextlib
-import glob
 import hashlib
 import json
 import os
@@ -77,15 +76,18 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def kernel_sources_sha16():
-    """Hash of the HIP / C++ sources the library is built from; the counter
-    figures in profiles/traffic.json carry the hash they were measured with."""
+TRAVERSAL_SOURCES = ('traverse.hip', 'search_lists.h', 'device_common.h')
+
+
+def kernel_sources_sha16(names=TRAVERSAL_SOURCES):
+    """Hash of the sources a kernel is compiled from (default: the traversal
+    kernel's); the counter figures in profiles/traffic.json carry the hash
+    they were measured with."""
     h = hashlib.sha256()
-    for path in sorted(glob.glob(os.path.join(ROOT, 'pilotann_amd', 'csrc', '*'))):
-        if path.endswith(('.hip', '.h', '.cpp')):
-            h.update(os.path.basename(path).encode())
-            with open(path, 'rb') as f:
-                h.update(f.read())
+    for name in names:
+        h.update(name.encode())
+        with open(os.path.join(ROOT, 'pilotann_amd', 'csrc', name), 'rb') as f:
+            h.update(f.read())
     return h.hexdigest()[:16]
 
 
@@ -236,7 +238,7 @@ def algorithmic_bytes(counters, B, dp, n_init):
             + C * (w + 4 * dp) + R * (w + 4))
 
 
-def measured_traffic(key):
+def measured_traffic(key, sources=TRAVERSAL_SOURCES):
     """Bytes per launch that left the L2 towards the fabric, from the
     rocprofv3 counter runs summarised under profiles/ (FETCH_SIZE and
     WRITE_SIZE, each scaled by what a plain copy of known size reads on the
@@ -252,7 +254,7 @@ def measured_traffic(key):
     if not entry:
         return None, None
     return (entry.get('hbm_bytes_per_launch'),
-            entry.get('kernel_sources_sha16') == kernel_sources_sha16())
+            entry.get('kernel_sources_sha16') == kernel_sources_sha16(sources))
 
 
 def time_stage(stage, ef, steps, warmup):
@@ -763,6 +765,9 @@ def device_refine_figures(cfg, index, stage, query, target, ef, host_top=None,
                   'admitted', 'completed', 'adjacency_entries'],
                  counters.cpu().tolist()))
     n_cand = cand_I.size(1)
+    refine_traffic = measured_traffic(
+        f'{cfg["name"]}/n={cfg["n"]}/queries={B}/ef={ef}/refine',
+        ('refine.hip', 'search_lists.h', 'device_common.h'))
     # query + candidates read + completed tails + adjacency ids + full rows
     # (4-byte id each) + buffer and top-k written
     nbytes = (B * 4 * d + B * n_cand * 8 + c['completed'] * 4 * (d - dp)
@@ -777,8 +782,8 @@ def device_refine_figures(cfg, index, stage, query, target, ef, host_top=None,
         'refine_kernel_ms': round(ms, 3),
         'refine_counters': c,
         'refine_algorithmic_bytes': int(nbytes),
-        'refine_hbm_traffic': measured_traffic(
-            f'{cfg["name"]}/n={cfg["n"]}/queries={B}/ef={ef}/refine')[0],
+        'refine_hbm_traffic': refine_traffic[0],
+        'refine_traffic_kernel_sources_unchanged': refine_traffic[1],
         'refine_achieved_GBps': round(nbytes / (ms * 1e-3) / 1e9, 1),
         'refine_frac_of_hbm_peak': round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
 
