@@ -108,6 +108,9 @@ def test_routing_random_shapes(seed, device):
 @pytest.mark.parametrize('B,d,n_out', [
     (1, 8, 8), (31, 64, 32), (64, 96, 64), (100, 200, 40), (1000, 768, 128),
     (257, 768, 768), (65, 72, 1),
+    # enough workgroups for the 64 x 128 and the 128 x 128 tiles, with ragged
+    # edges in all three dimensions
+    (3300, 1000, 1000), (6437, 1000, 1000),
 ])
 def test_rotation_matches_float64_matmul(B, d, n_out, device):
     """`pa_rotate` (query @ VT.T, first n_out columns) against a float64
@@ -122,7 +125,7 @@ def test_rotation_matches_float64_matmul(B, d, n_out, device):
     out = kernels.rotate(query.to(device), VT.to(device), n_out)
     torch.cuda.synchronize()
     assert out.shape == (B, n_out)
-    ref = (query.double() @ VT.double().T)[:, :n_out]
+    ref = (query.to(device).double() @ VT.to(device).double().T)[:, :n_out].cpu()
     bound = 4 * d * 2.0 ** -24 * query.double().norm(dim=1, keepdim=True) \
         * VT.double().norm(dim=1)[:n_out].unsqueeze(0)
     assert bool(((out.cpu().double() - ref).abs() <= bound).all())
