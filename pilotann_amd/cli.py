@@ -12,9 +12,11 @@ faiss on the CPU, is not available here; its role — the search without a GPU
 — is played by the library's host search on the full graph
 (``host-cpu: recall=…, duration=…ms``).
 
-Datasets are synthetic (the reference's files are not distributable):
-``synth:<n>x<d>[:<centres>[:<spectrum exponent>]]``, a unit-norm Gaussian
-mixture; the default is the shape of the headline benchmark
+Datasets: the reference's names (``deep-1m``, ``text2img-10m``, ``wiki-1m``,
+``laion-1m``, ``fuzz-64k`` …, read by ``utils.DataLoader`` from
+``--data_root``, default ``.dataset`` as in the reference), or a synthetic
+unit-norm Gaussian mixture, ``synth:<n>x<d>[:<centres>[:<spectrum
+exponent>]]``; the default is the shape of the headline benchmark
 (``synth:1000000x768:1024:0.5`` with ``--d_principle 128 --n_neighbors 64
 --router router64x64``).
 
@@ -36,9 +38,6 @@ QUERY_POOL = 4096         # utils/loader.py:10
 def parse_dataset(name: str):
     """``synth:<n>x<d>[:<centres>[:<spectrum exponent>]]`` -> generator
     arguments (unit-norm mixture, sigma 1, seed 7)."""
-    if not name.startswith('synth:'):
-        raise SystemExit(f'unknown dataset {name!r}: '
-                         'synth:<n>x<d>[:<centres>[:<spectrum exponent>]]')
     parts = name[len('synth:'):].split(':')
     n, d = (int(v) for v in parts[0].lower().split('x'))
     centres = int(parts[1]) if len(parts) > 1 else 64
@@ -51,8 +50,8 @@ class Profiler:
     """``ANNProfiler`` of ``script/common.py:21-197`` for this library."""
 
     def __init__(self, dataset, algorithm, n_queries, d_principle,
-                 entry_method, sample_ratio, device, refine='host'):
-        self.spec = parse_dataset(dataset)
+                 entry_method, sample_ratio, device, refine='host',
+                 data_root='.dataset', seed=7):
         self.algorithm = algorithm
         self.n_queries = n_queries
         self.d_principle = d_principle
@@ -60,18 +59,34 @@ class Profiler:
         self.sample_ratio = sample_ratio
         self.device = device
         self.refine = refine
+        self.seed = seed
         self.index = None
         self.method = None
-        s = self.spec
-        print('[{}] dataset: {}, d_model: {}'.format(algorithm, dataset, s['d']))
-        kw = dict(normalize=s['normalize'], device=device, decay=s['decay'])
-        self.storage = utils.gaussian_mixture(
-            s['n'], s['d'], s['n_centers'], s['sigma'], seed=s['seed'], **kw)
-        self.queries = utils.gaussian_mixture(
-            QUERY_POOL, s['d'], s['n_centers'], s['sigma'], seed=s['seed'] + 1,
-            center_seed=s['seed'], **kw)
+        self.loader = None
         self.targets = {}
-        self.draw = torch.Generator().manual_seed(s['seed'] + 2)
+        self.draw = torch.Generator().manual_seed(seed + 2)
+        if dataset.startswith('synth:'):
+            s = parse_dataset(dataset)
+            kw = dict(normalize=s['normalize'], device=device, decay=s['decay'])
+            self.storage = utils.gaussian_mixture(
+                s['n'], s['d'], s['n_centers'], s['sigma'], seed=s['seed'], **kw)
+            self.queries = utils.gaussian_mixture(
+                QUERY_POOL, s['d'], s['n_centers'], s['sigma'], seed=s['seed'] + 1,
+                center_seed=s['seed'], **kw)
+        else:
+            try:
+                self.loader = utils.DataLoader(dataset, root=data_root, seed=seed,
+                                               device=device)
+            except NotImplementedError:
+                raise SystemExit(
+                    f'unknown dataset {dataset!r}: a name of the reference '
+                    '(deep-1m, text2img-1m, wiki-1m, laion-1m, fuzz-64k, ...) or '
+                    'synth:<n>x<d>[:<centres>[:<spectrum exponent>]]')
+            self.storage = self.loader.load_storage()
+            if self.storage is None:
+                raise SystemExit(f'{dataset}: no base vectors under {data_root}')
+        print('[{}] dataset: {}, d_model: {}'.format(
+            algorithm, dataset, self.storage.size(-1)))
 
     def target(self, k):
         if k not in self.targets:
@@ -80,6 +95,8 @@ class Profiler:
         return self.targets[k]
 
     def load_query(self, k):
+        if self.loader is not None:
+            return self.loader.load_query(self.n_queries, k=k)
         pick = torch.randperm(QUERY_POOL, generator=self.draw)[:self.n_queries]
         return self.queries[pick.to(self.queries.device)].cpu(), self.target(k)[pick]
 
@@ -89,9 +106,9 @@ class Profiler:
             return          # both methods search the same index
         prefix = {'hnsw': 'nsw', 'nsg': 'nsg'}[self.algorithm]
         index = layers.IndexStaged(
-            d_model=self.spec['d'], d_principle=self.d_principle,
+            d_model=self.storage.size(-1), d_principle=self.d_principle,
             sample_ratio=self.sample_ratio, entry_method=self.entry_method,
-            graph_method=f'{prefix}{n_neighbors}', seed=self.spec['seed'],
+            graph_method=f'{prefix}{n_neighbors}', seed=self.seed,
             build_device=self.device)
         index.train(self.storage)
         index.to(self.device)
@@ -143,6 +160,8 @@ def main(argv=None):
     parser.add_argument('--router', type=str, default='router64x64')
     parser.add_argument('--dataset', type=str,
                         default='synth:1000000x768:1024:0.5')
+    parser.add_argument('--data_root', default='.dataset',
+                        help="directory of the reference's dataset folders")
     parser.add_argument('--refine', choices=['host', 'device'], default='host',
                         help="where stages 2 and 3 run (the reference: host)")
     parser.add_argument('--methods', type=lambda s: s.split(','),
@@ -160,7 +179,8 @@ def main(argv=None):
                         entry_method=args.router,
                         sample_ratio=args.sample_ratio,
                         d_principle=args.d_principle, n_queries=args.n_queries,
-                        device=args.device, refine=args.refine)
+                        device=args.device, refine=args.refine,
+                        data_root=args.data_root)
     if args.load:
         profiler.load(args.load)
     records = {method: [] for method in args.methods}

@@ -15,9 +15,11 @@ from .graphs import (knn_graph, graph_init, subgraph_init, graph_sampling,
 from .router import router_init
 from .synth import gaussian_mixture, brute_force_topk
 from .layout import locality_order
+from .search import search_simple
+from .loader import DataLoader
 
 __all__ = [
     'recall', 'svd', 'knn_graph', 'graph_init', 'subgraph_init',
     'graph_sampling', 'connect_graph', 'reachable', 'router_init', 'gaussian_mixture', 'brute_force_topk',
-    'locality_order',
+    'locality_order', 'search_simple', 'DataLoader',
 ]

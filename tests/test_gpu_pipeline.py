@@ -145,3 +145,34 @@ def test_command_line_benchmark_prints_the_reference_lines(device, capsys):
     assert [r['ef_search'] for r in records['search-pilot']] == [16, 32]
     # more effort, better recall
     assert records['search-pilot'][1]['recall'] >= records['search-pilot'][0]['recall']
+
+
+def test_command_line_benchmark_reads_the_reference_dataset_layout(device, capsys, tmp_path):
+    """`--dataset deep-1m` as script/bench_1.py:32-34 passes it on: base,
+    queries and ground truth in the .fbin / .ibin layout of
+    pilot_ann/utils/loader.py:43-50,92-148 under the data root."""
+    import os
+    import re
+    import numpy as np
+    from pilotann_amd import cli, utils
+    from pilotann_amd.utils.loader import write_bins
+    base = utils.gaussian_mixture(20000, 64, 16, 1.0, seed=3, normalize=True, decay=0.5)
+    query = utils.gaussian_mixture(512, 64, 16, 1.0, seed=4, center_seed=3,
+                                   normalize=True, decay=0.5)
+    truth = utils.brute_force_topk(query, base, 100)
+    folder = tmp_path / 'deep-1m'
+    os.makedirs(folder)
+    write_bins(folder / 'base.fbin', base.numpy())
+    write_bins(folder / 'query.fbin', query.numpy())
+    write_bins(folder / 'groundtruth.ibin', truth.numpy().astype(np.int32))
+    records = cli.main(['--dataset', 'deep-1m', '--data_root', str(tmp_path),
+                        '--d_principle', '32', '--n_neighbors', '32',
+                        '--router', 'router16x32', '--ef_search', '32',
+                        '--n_queries', '256', '--n_repeats', '2',
+                        '--methods', 'search-pilot', '--device', str(device)])
+    out = capsys.readouterr().out
+    assert '[hnsw] dataset: deep-1m, d_model: 64' in out
+    assert re.search(r'^search-pilot: recall=\d\.\d{3}, duration=\d+\.\d{3}ms$', out, flags=re.M)
+    assert records['search-pilot'][0]['recall'] > 0.7
+    with pytest.raises(SystemExit):
+        cli.main(['--dataset', 'sift-1m', '--device', str(device)])
