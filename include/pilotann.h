@@ -237,6 +237,42 @@ int pa_traverse_refine(int64_t *out_I, float *out_D, int64_t *buf_I,
                        int n_init, int n_buffers, int k, int ef_search);
 
 /*
+ * The reference's operator hooks (extension/ops_cpu.cpp:8-95,
+ * pilot_ann/kernels/__init__.py:5-35): one call of a heap primitive of
+ * extension/inc/heapq.cuh on a host array heap of n (key, value) cells, a set
+ * of visited marks, and the row distance of extension/inc/distance.h.  Host
+ * pointers; the code is the one pa_traverse_cpu runs.
+ *
+ * pa_heapq_pop: heapq_pop_cpu (:8-13) - the root is dropped, (inf, -1) sinks
+ * from its place.  pa_heapq_pushpop: heapq_pushpop_cpu (:15-24) - a key larger
+ * than the root replaces it and sinks.  pa_heapq_replace: heapq_replace_cpu
+ * (:26-35) - a key smaller than the leaf reached through the larger children
+ * overwrites that leaf and rises.
+ */
+int pa_heapq_pop(float *keys, int64_t *values, int64_t n);
+int pa_heapq_pushpop(float *keys, int64_t *values, int64_t n, float key,
+                     int64_t value);
+int pa_heapq_replace(float *keys, int64_t *values, int64_t n, float key,
+                     int64_t value);
+
+/*
+ * bitmask_put_cpu (ops_cpu.cpp:37-51, extension/inc/bitmask.hpp:11-46): marks
+ * [n] := 0, then the first marker (1) at every key.  Keys outside [0, n) are
+ * refused with PA_E_RANGE before anything is written.
+ */
+int pa_bitmask_put(int32_t *marks, int64_t n, const int64_t *keys,
+                   int64_t n_keys);
+
+/*
+ * square_dist_cpu (ops_cpu.cpp:53-85): out[i] = squared L2 distance between
+ * query [d_model] and row nodelist[i] of storage [n_storage * d_model], in the
+ * summation order of distance.h:31-55.  d_model % 8 == 0.
+ */
+int pa_square_dist(float *out, const float *query, const float *storage,
+                   const int64_t *nodelist, int64_t n_nodes, int64_t n_storage,
+                   int d_model);
+
+/*
  * Replaces `pipeline` (extension/pipeline_cpu.cpp:32-145,
  * pilot_ann/kernels/__init__.py:106-124): splits the batch into chunks, runs
  * pa_traverse for chunk i+1 and i+2 on two internal streams while

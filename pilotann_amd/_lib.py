@@ -35,6 +35,11 @@ _SIGNATURES = {
     'pa_traverse_refine': (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                                   _vp, _vp, _vp, _vp, _i64, _i64, _int, _int,
                                   _int, _int, _int, _int]),
+    'pa_heapq_pop': (_int, [_vp, _vp, _i64]),
+    'pa_heapq_pushpop': (_int, [_vp, _vp, _i64, ctypes.c_float, _i64]),
+    'pa_heapq_replace': (_int, [_vp, _vp, _i64, ctypes.c_float, _i64]),
+    'pa_bitmask_put': (_int, [_vp, _i64, _vp, _i64]),
+    'pa_square_dist': (_int, [_vp, _vp, _vp, _vp, _i64, _i64, _int]),
     'pa_rows_prepare': (_int, [_vp, _vp, _i64, _int, _vp]),
     'pa_refine_plan': (_int, [_i64, _i64, _int, _int,
                               ctypes.POINTER(_int), ctypes.POINTER(_sz)]),

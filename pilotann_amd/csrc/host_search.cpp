@@ -304,3 +304,79 @@ extern "C" int pa_traverse_refine(
     }
     return PA_OK;
 }
+
+// ---- the reference's operator hooks (extension/ops_cpu.cpp:8-95) -------------
+//
+// pilot_ann/kernels/__init__.py:5-35 exposes the heap primitives, the visited
+// marks and the row distance of the host search one call at a time; the
+// reference's operator tests (test/kernel/test_operators.py) are written
+// against them.  These run the same code the searches above run.
+
+namespace {
+bool heap_args_ok(const float *keys, const int64_t *values, int64_t n) {
+    return keys && values && n >= 1 && n < (1ll << 31);
+}
+}  // namespace
+
+// heapq_pop_cpu, ops_cpu.cpp:8-13: the root leaves, (inf, -1) takes its place.
+extern "C" int pa_heapq_pop(float *keys, int64_t *values, int64_t n) {
+    if (n == 0) return PA_OK;
+    if (!heap_args_ok(keys, values, n)) return n < 0 || n >= (1ll << 31) ? PA_E_SHAPE : PA_E_NULL;
+    float k;
+    int64_t v;
+    HeapView{keys, values, (int)n}.pop(&k, &v);
+    return PA_OK;
+}
+
+// heapq_pushpop_cpu, ops_cpu.cpp:15-24.
+extern "C" int pa_heapq_pushpop(float *keys, int64_t *values, int64_t n,
+                                float key, int64_t value) {
+    if (n == 0) return PA_OK;
+    if (!heap_args_ok(keys, values, n)) return n < 0 || n >= (1ll << 31) ? PA_E_SHAPE : PA_E_NULL;
+    HeapView{keys, values, (int)n}.pushpop(key, value);
+    return PA_OK;
+}
+
+// heapq_replace_cpu, ops_cpu.cpp:26-35.
+extern "C" int pa_heapq_replace(float *keys, int64_t *values, int64_t n,
+                                float key, int64_t value) {
+    if (n == 0) return PA_OK;
+    if (!heap_args_ok(keys, values, n)) return n < 0 || n >= (1ll << 31) ? PA_E_SHAPE : PA_E_NULL;
+    HeapView{keys, values, (int)n}.replace(key, value);
+    return PA_OK;
+}
+
+// bitmask_put_cpu, ops_cpu.cpp:37-51: a fresh set of n visited marks (all
+// zero), advanced once, with the marker written at every key.  A key outside
+// [0, n) is an error here (the reference writes out of bounds).
+extern "C" int pa_bitmask_put(int32_t *marks, int64_t n, const int64_t *keys,
+                              int64_t n_keys) {
+    if (n < 0 || n_keys < 0) return PA_E_SHAPE;
+    if ((n && !marks) || (n_keys && !keys)) return PA_E_NULL;
+    for (int64_t i = 0; i < n_keys; ++i)
+        if (keys[i] < 0 || keys[i] >= n) return PA_E_RANGE;
+    std::memset(marks, 0, (size_t)n * sizeof(int32_t));
+    const int32_t marker = 1;  // bitmask.hpp:16-31: the first marker
+    for (int64_t i = 0; i < n_keys; ++i) marks[keys[i]] = marker;
+    return PA_OK;
+}
+
+// square_dist_cpu, ops_cpu.cpp:53-85: squared L2 distance of the query to the
+// rows nodelist[i] of storage, four rows at a time while more than four are
+// left, then one by one (both forms add in the same order).
+extern "C" int pa_square_dist(float *out, const float *query,
+                              const float *storage, const int64_t *nodelist,
+                              int64_t n_nodes, int64_t n_storage, int d_model) {
+    if (n_nodes < 0 || n_storage < 0) return PA_E_SHAPE;
+    if (d_model <= 0 || d_model % 8) return PA_E_DIM;
+    if (n_nodes == 0) return PA_OK;
+    if (!out || !query || !storage || !nodelist) return PA_E_NULL;
+    for (int64_t i = 0; i < n_nodes; ++i)
+        if (nodelist[i] < 0 || nodelist[i] >= n_storage) return PA_E_RANGE;
+    int64_t at = 0;
+    for (; at + kTile < n_nodes; at += kTile)
+        square_dist4(out + at, query, storage, nodelist + at, d_model);
+    for (; at < n_nodes; ++at)
+        out[at] = square_dist(query, storage + nodelist[at] * (int64_t)d_model, d_model);
+    return PA_OK;
+}

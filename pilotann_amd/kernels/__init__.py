@@ -298,6 +298,79 @@ def entry_distances(query: torch.Tensor, entry_vectors: torch.Tensor):
     return distances
 
 
+# ---- the reference's operator hooks ------------------------------------------
+
+def _heap(keys, values):
+    _check(keys, 'keys', 1, torch.float32, False)
+    _check(values, 'values', 1, torch.int64, False)
+    _require(keys.numel() == values.numel(), 'keys.numel() == values.numel()')
+
+
+def heapq_pop(keys: torch.Tensor, values: torch.Tensor):
+    """``kernels.heapq_pop`` (``pilot_ann/kernels/__init__.py:5-7``,
+    ``ops_cpu.cpp:8-13``): drops the root of the array heap in place."""
+    _heap(keys, values)
+    _lib.check(_lib.lib().pa_heapq_pop(_ptr(keys), _ptr(values), keys.numel()),
+               'pa_heapq_pop')
+
+
+def heapq_pushpop(keys: torch.Tensor, values: torch.Tensor, key: float, value: int):
+    """``kernels.heapq_pushpop`` (``pilot_ann/kernels/__init__.py:10-15``,
+    ``ops_cpu.cpp:15-24``), in place."""
+    _heap(keys, values)
+    _lib.check(_lib.lib().pa_heapq_pushpop(
+        _ptr(keys), _ptr(values), keys.numel(), float(key), int(value)),
+        'pa_heapq_pushpop')
+
+
+def heapq_replace(keys: torch.Tensor, values: torch.Tensor, key: float, value: int):
+    """``kernels.heapq_replace`` (``pilot_ann/kernels/__init__.py:18-23``,
+    ``ops_cpu.cpp:26-35``), in place."""
+    _heap(keys, values)
+    _lib.check(_lib.lib().pa_heapq_replace(
+        _ptr(keys), _ptr(values), keys.numel(), float(key), int(value)),
+        'pa_heapq_replace')
+
+
+def bitmask_put(keys: torch.Tensor, n: int):
+    """``kernels.bitmask_put`` (``pilot_ann/kernels/__init__.py:26-27``,
+    ``ops_cpu.cpp:37-51``): int32 marks of ``n`` nodes, non-zero at ``keys``."""
+    _check(keys, 'keys', 1, torch.int64, False)
+    marks = torch.empty(int(n), dtype=torch.int32)
+    _lib.check(_lib.lib().pa_bitmask_put(_ptr(marks), int(n), _ptr(keys),
+                                         keys.numel()), 'pa_bitmask_put')
+    return marks
+
+
+def square_dist(query: torch.Tensor, storage: torch.Tensor, nodelist: torch.Tensor):
+    """``kernels.square_dist`` (``pilot_ann/kernels/__init__.py:30-35``,
+    ``ops_cpu.cpp:53-85``): squared L2 distances between ``query`` and the
+    rows ``nodelist`` of ``storage``, host tensors."""
+    _check(query, 'query', 1, torch.float32, False)
+    _check(storage, 'storage', 2, torch.float32, False)
+    _check(nodelist, 'nodelist', 1, torch.int64, False)
+    _require(storage.size(-1) == query.size(0), 'storage.size(-1) == d_model')
+    output = torch.zeros(nodelist.size(0), dtype=torch.float32)
+    _lib.check(_lib.lib().pa_square_dist(
+        _ptr(output), _ptr(query), _ptr(storage), _ptr(nodelist),
+        nodelist.size(0), storage.size(0), query.size(0)), 'pa_square_dist')
+    return output
+
+
+def graph_sampling(indptr: torch.Tensor, indices: torch.Tensor, n_samples: int,
+                   n_hops: int, seed: int = None):
+    """``kernels.graph_sampling`` (``pilot_ann/kernels/__init__.py:38-44``,
+    ``extension/sampling_cpu.cpp:5-65``): seed nodes and everything within
+    ``n_hops`` edges of them until ``n_samples`` nodes are in; returns
+    ``[nodelist, mapping]`` as lists.  The reference seeds its draws with the
+    time; ``seed=None`` does the same, a number makes the sample repeatable."""
+    import time
+    from ..utils.graphs import graph_sampling as sample
+    nodelist, mapping = sample(indptr, indices, n_samples=n_samples, n_hops=n_hops,
+                               seed=int(time.time()) if seed is None else seed)
+    return [nodelist.tolist(), mapping.tolist()]
+
+
 # ---- host stages ------------------------------------------------------------
 
 def traverse_cpu(output_I: torch.Tensor,
