@@ -105,8 +105,55 @@ def make_data(cfg, device):
     return x, q, target
 
 
-def build_index(cfg, device):
+def save_stage_cache(path, cfg, index, q, target):
+    """What the device stage of a `stage_only` configuration needs, so that a
+    counter run does not pay for the index build again: rotation, sample,
+    subgraph, router, queries, ground truth and the sampled rows' first
+    d_principle coordinates."""
+    torch.save({
+        'config': {k: v for k, v in cfg.items() if k != 'name'},
+        'VT': index.VT, 'nodelist': index.nodelist, 'mapping': index.mapping,
+        'subgraph.indptr': index.subgraph.indptr,
+        'subgraph.indices': index.subgraph.indices,
+        'entry': index.entry.state_dict(),
+        'rows': index.storage[index.nodelist][:, :cfg['dp']].contiguous(),
+        'query': q, 'target': target,
+    }, path)
+
+
+def load_stage_cache(path, cfg, device):
     from pilotann_amd import IndexStaged
+    from pilotann_amd.layers.staged import GraphModule
+    saved = torch.load(path, weights_only=True)
+    if saved['config'] != {k: v for k, v in cfg.items() if k != 'name'}:
+        raise SystemExit(f'{path} was written for another configuration')
+    index = IndexStaged(d_model=cfg['d'], d_principle=cfg['dp'],
+                        sample_ratio=cfg['ratio'], graph_method=cfg['graph'],
+                        entry_method=cfg['entry'], seed=cfg['seed'],
+                        build_device=device)
+    for name in ['VT', 'nodelist', 'mapping']:
+        index.register_buffer(name, saved[name])
+    index.register_module('subgraph', GraphModule(
+        saved['subgraph.indptr'], saved['subgraph.indices']))
+    for name, value in saved['entry'].items():
+        index.entry.register_buffer(name, value)
+    # the rows the stage reads, at their global positions; the others (and the
+    # coordinates past d_principle) are never looked at by the device stage
+    storage = torch.zeros(cfg['n'], cfg['dp'])
+    storage[saved['nodelist']] = saved['rows']
+    index.register_buffer('storage', storage)
+    index.fullgraph = None
+    index.to(device)
+    return index, saved['query'], saved['target']
+
+
+def build_index(cfg, device, stage_cache=None):
+    from pilotann_amd import IndexStaged
+    if stage_cache and os.path.exists(stage_cache):
+        t0 = time.time()
+        out = load_stage_cache(stage_cache, cfg, device)
+        log(f'[bench] index read from {stage_cache} {time.time() - t0:.1f}s')
+        return out
     t0 = time.time()
     x, q, target = make_data(cfg, device)
     log(f'[bench] data + ground truth {time.time() - t0:.1f}s')
@@ -124,6 +171,9 @@ def build_index(cfg, device):
     index.to(device)
     log(f'[bench] index built {time.time() - t0:.1f}s, '
         f'sampled {index.nodelist.numel()} of {cfg["n"]}')
+    if stage_cache:
+        save_stage_cache(stage_cache, cfg, index, q.cpu(), target)
+        log(f'[bench] stage inputs written to {stage_cache}')
     return index, q.cpu(), target
 
 
@@ -481,6 +531,11 @@ def main():
                          'device and the refine kernel alone (needs --ef), '
                          'print those figures and exit; with --no-context '
                          'the refine kernel alone (4 launches)')
+    ap.add_argument('--stage-cache', default=None, metavar='FILE',
+                    help='configurations that build the device stage only '
+                         '(c5): write the stage\'s inputs to FILE after the '
+                         'build, or read them from FILE if it exists (for '
+                         'counter runs, which slow the build down)')
     ap.add_argument('--copy-calibration', action='store_true',
                     help='only run a plain 1 GiB device copy five times (to '
                          'scale the FETCH_SIZE / WRITE_SIZE counters) and exit')
@@ -514,7 +569,10 @@ def main():
         cfg['decay'] = args.decay
     device = 'cuda:0'
     torch.cuda.set_device(0)
-    index, query, target = build_index(cfg, device)
+    if args.stage_cache and not cfg.get('stage_only'):
+        ap.error('--stage-cache is for configurations that build the device '
+                 'stage only')
+    index, query, target = build_index(cfg, device, args.stage_cache)
     stage = Stage(index, query, device)
     B, k, dp = stage.B, cfg['k'], cfg['dp']
 
