@@ -141,6 +141,7 @@ __global__ __launch_bounds__(kWave) PA_REFINE_OCCUPANCY(H) void refine_kernel(Re
     int *oval = reinterpret_cast<int *>(okey + kHeapCells);
     OpenList<H> open;
     open.cells = lds.heap;
+    open.deep = nullptr;  // the whole list in registers and LDS
     int *cand_id = lds.cand_id;
     float *cand_key = lds.cand_key;
     const int d = a.d;

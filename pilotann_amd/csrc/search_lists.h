@@ -28,7 +28,11 @@ constexpr int kSeenCache = 1 << kSeenCacheLog2;  // LDS words remembering visite
 // in lane j), bank B level 6 (lane j - 64), banks C and D the left and right
 // children of level 7 (lane (j - 128) / 2), so a sibling pair is always two
 // v_readlane of known registers.  Deeper nodes sit in LDS at [j - 256] as
-// (key, value), a sibling pair per aligned 16 bytes.  Keys are kept as
+// (key, value), a sibling pair per aligned 16 bytes; with DEEP the levels
+// from DEEP on sit in device memory instead (the wavefront's own region, at
+// [j - 2^DEEP], same cells): a long list then takes less LDS, more
+// wavefronts fit a compute unit, and a walk pays one memory round trip per
+// such level.  Keys are kept as
 // order-preserving integers (float_to_key) so that every comparison of a walk
 // is a scalar integer compare.  All lanes run the same, uniform, control flow; the walks
 // are unrolled by level so that each level is a dozen instructions.  After
@@ -66,28 +70,46 @@ __device__ __forceinline__ int add_if_bit(int c, unsigned long long mask, int id
     return r;
 }
 
-template <int H>
+// Cells of an open list of 2H cells that sit in device memory when the levels
+// from `deep` on do (0: none do).
+constexpr int open_list_deep_cells(int H, int deep) {
+    return deep >= 8 && deep <= floor_log2(2 * H) ? 2 * H + 2 - (1 << deep) : 0;
+}
+
+template <int H, int DEEP = 0>
 struct OpenList {
     static constexpr int kSize = 2 * H;           // cells of the reference heap
     static constexpr int kDepth = floor_log2(kSize);  // deepest level
     static constexpr int kRegNodes = 256;
-    static constexpr int kLdsCells = kSize + 2 > kRegNodes ? kSize + 2 - kRegNodes : 0;
+    static constexpr int kDeepCells = open_list_deep_cells(H, DEEP);
+    static constexpr int kDeepFrom = kDeepCells ? DEEP : kDepth + 1;
+    static constexpr int kDeepBase = 1 << kDeepFrom;  // first node in device memory
+    static constexpr int kLdsCells =
+        kDeepCells ? kDeepBase - kRegNodes
+                   : (kSize + 2 > kRegNodes ? kSize + 2 - kRegNodes : 0);
     static constexpr int kInf = 0x7f800000;       // float_to_key(+inf)
     int Ak, Av, Bk, Bv, Ck, Cv, Dk, Dv;
-    int2 *cells;  // node j >= 256 at [j - 256] as (key, value); 16-byte aligned
+    int2 *cells;  // node j in [256, kDeepBase) at [j - 256] as (key, value); 16-byte aligned
+    int2 *deep;   // node j >= kDeepBase at [j - kDeepBase], device memory, 16-byte aligned
+    int4 pending;   // pop(): the requested pair of level kDeepFrom, until pop_finish()
+    int pending_j;  // its parent, 0 = nothing pending (uniform)
 
     __device__ __forceinline__ static int rl(int x, int l) {
         return __builtin_amdgcn_readlane(x, l);
     }
-    // storage class of a level: 0 bank A, 1 bank B, 2 banks C/D, 3 LDS
+    // storage class of a level: 0 bank A, 1 bank B, 2 banks C/D, 3 LDS,
+    // 4 device memory
     __device__ __forceinline__ static constexpr int kind(int level) {
-        return level <= 5 ? 0 : level == 6 ? 1 : level == 7 ? 2 : 3;
+        return level <= 5 ? 0 : level == 6 ? 1 : level == 7 ? 2
+                                           : level < kDeepFrom ? 3 : 4;
     }
 
     __device__ __forceinline__ void reset(int lane) {
         Ak = Bk = Ck = Dk = kInf;
         Av = Bv = Cv = Dv = -1;
         for (int i = lane; i < kLdsCells; i += kWave) cells[i] = make_int2(kInf, -1);
+        for (int i = lane; i < kDeepCells; i += kWave) deep[i] = make_int2(kInf, -1);
+        pending_j = 0;
     }
 
     // keys (and values) of the sibling pair (c, c + 1), c even, of a level.
@@ -108,7 +130,9 @@ struct OpenList {
             if (VALS) va = rl(Cv, l), vb = rl(Dv, l);
         } else {
             // one 16-byte read: both children with their values
-            const int4 p = *reinterpret_cast<const int4 *>(cells + (c - kRegNodes));
+            const int4 p = KIND == 3
+                ? *reinterpret_cast<const int4 *>(cells + (c - kRegNodes))
+                : *reinterpret_cast<const int4 *>(deep + (c - kDeepBase));
             if (VALS) va = uni(p.y), vb = uni(p.w);
             ka = uni(p.x), kb = uni(p.z);
         }
@@ -123,7 +147,7 @@ struct OpenList {
             const int left = rl(Ck, l), right = rl(Dk, l);
             return (j & 1) ? right : left;
         }
-        return uni(cells[j - kRegNodes].x);
+        return uni(KIND == 3 ? cells[j - kRegNodes].x : deep[j - kDeepBase].x);
     }
     __device__ __forceinline__ int val_of(const int KIND, int j) const {
         if (KIND == 0) return rl(Av, j);
@@ -133,7 +157,7 @@ struct OpenList {
             const int left = rl(Cv, l), right = rl(Dv, l);
             return (j & 1) ? right : left;
         }
-        return uni(cells[j - kRegNodes].y);
+        return uni(KIND == 3 ? cells[j - kRegNodes].y : deep[j - kDeepBase].y);
     }
     // lane l of a key bank and of its value bank := two uniform values
     // (v_writelane takes one scalar register besides M0, which holds the lane)
@@ -163,10 +187,12 @@ struct OpenList {
             Cv = (here && !right) ? v : Cv;
             Dk = (here && right) ? k : Dk;
             Dv = (here && right) ? v : Dv;
-        } else {
+        } else if (KIND == 3) {
             // every lane stores the same pair to the same cell: one LDS
             // write, and no divergent branch around it
             cells[j - kRegNodes] = make_int2(k, v);
+        } else {
+            deep[j - kDeepBase] = make_int2(k, v);
         }
     }
 
@@ -266,14 +292,52 @@ struct OpenList {
             put(kind(L - 1), node[L - 1], ck[L], cv[L], lane);
         }
         int j = node[kRegLevels];
+        pending_j = 0;
 #pragma unroll
         for (int L = kRegLevels + 1; L <= kDepth; ++L) {
             if (L == kDepth && 2 * j > kSize) {
                 put(kind(L - 1), j, kInf, -1, lane);
                 return;
             }
+            if (kDeepCells && L == kDeepFrom) {
+                // the pair is requested; pop_finish() goes on from here
+                pending = *reinterpret_cast<const int4 *>(deep + (2 * j - kDeepBase));
+                pending_j = j;
+                return;
+            }
             int ka, kb, va, vb;
-            pair(3, true, 2 * j, ka, kb, va, vb);
+            pair(kind(L), true, 2 * j, ka, kb, va, vb);
+            if (L == kDepth) kb = 2 * j == kSize ? ka : kb;
+            const int k = min(ka, kb);
+            const int v = k != ka ? vb : va;
+            const int c = add_if_ne(2 * j, k, ka);
+            put(kind(L - 1), j, k, v, lane);
+            j = c;
+        }
+        put(kind(kDepth), j, kInf, -1, lane);
+    }
+    // The levels of a pop that sit in device memory.  pop() only requests the
+    // first pair it needs from there; the caller puts the work that does not
+    // touch the list (the root is in registers) between the two, and calls
+    // this before the next walk or pop.  Nothing to do without such levels.
+    __device__ __forceinline__ void pop_finish(int lane) {
+        if (!kDeepCells) return;
+        int j = pending_j;
+        if (j == 0) return;
+        pending_j = 0;
+#pragma unroll
+        for (int L = kDeepFrom; L <= kDepth; ++L) {
+            if (L == kDepth && 2 * j > kSize) {
+                put(kind(L - 1), j, kInf, -1, lane);
+                return;
+            }
+            int ka, kb, va, vb;
+            if (L == kDeepFrom) {
+                ka = uni(pending.x), va = uni(pending.y);
+                kb = uni(pending.z), vb = uni(pending.w);
+            } else {
+                pair(kind(L), true, 2 * j, ka, kb, va, vb);
+            }
             if (L == kDepth) kb = 2 * j == kSize ? ka : kb;
             const int k = min(ka, kb);
             const int v = k != ka ? vb : va;
@@ -309,7 +373,7 @@ struct OpenList {
                 j = (L == kDepth && 2 * j == kSize) ? 2 * j : step_down(L, j, ch);
             } else {
                 int ka, kb, va, vb;
-                pair(3, false, 2 * j, ka, kb, va, vb);
+                pair(kind(L), false, 2 * j, ka, kb, va, vb);
                 if (L == kDepth) kb = 2 * j == kSize ? ka : kb;
                 walked_key = max(ka, kb);
                 j = add_if_ne(2 * j, walked_key, ka);
@@ -319,9 +383,9 @@ struct OpenList {
         Leaf leaf;
         leaf.j = j, leaf.bottom = bottom;
         if (bottom)
-            leaf.key = kind(kDepth) == 3 ? walked_key : key_of(kind(kDepth), j);
+            leaf.key = kind(kDepth) >= 3 ? walked_key : key_of(kind(kDepth), j);
         else
-            leaf.key = kind(kDepth - 1) == 3 ? walked_key : key_of(kind(kDepth - 1), j);
+            leaf.key = kind(kDepth - 1) >= 3 ? walked_key : key_of(kind(kDepth - 1), j);
         return leaf;
     }
     // SPARSE: the heap is nearly empty (the entries of a query are pushed),

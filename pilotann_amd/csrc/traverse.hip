@@ -90,15 +90,38 @@ __global__ void reset_work_counter(int *counter) { *counter = 0; }
 #define PA_OCCUPANCY(H) __attribute__((amdgpu_waves_per_eu((H) <= 256 ? 4 : (H) <= 384 ? 3 : (H) <= 1024 ? 2 : 1, 8)))
 #endif
 
+// The longest open list (4096 cells) keeps its last two levels in the
+// wavefront's region of device memory instead of LDS (search_lists.h): first
+// level kept there, 0 = the whole list in registers and LDS.  Measured on
+// 10 000 queries over 500 000 rows of 128 floats: lists of 4096 cells run in
+// 50.0 instead of 69.7 ms with level 11 on in device memory (7 instead of 4
+// wavefronts per compute unit) and in 60.4 ms with level 10 on; lists of 2048
+// cells take 23.1 ms with level 10 on in device memory against 23.4 ms
+// without (11 instead of 8 wavefronts, each as much slower) and 29.6 ms with
+// level 9 on, so they stay in LDS.
+#ifndef PA_DEEP_512
+#define PA_DEEP_512 0
+#endif
+#ifndef PA_DEEP_1024
+#define PA_DEEP_1024 0
+#endif
+#ifndef PA_DEEP_2048
+#define PA_DEEP_2048 11
+#endif
+constexpr int deep_from(int H) {
+    return H == 2048 ? PA_DEEP_2048 : H == 1024 ? PA_DEEP_1024 : H == 512 ? PA_DEEP_512 : 0;
+}
+
 template <int H, int DP8>
 __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(TraverseArgs a) {
     // One static block, in this order: the compiler then knows every LDS
     // address, and a heap cell [j - 256] is the scalar j * 8 plus a positive
     // constant that fits the instruction's offset field.
+    using Open = OpenList<H, deep_from(H)>;
     constexpr int S = (H + kWave - 1) / kWave;
     constexpr int kSortN = H <= kWave ? kWave : 1 << (floor_log2(H - 1) + 1);
     constexpr int kHeapCells =
-        OpenList<H>::kLdsCells > kSortN ? OpenList<H>::kLdsCells : kSortN;
+        Open::kLdsCells > kSortN ? Open::kLdsCells : kSortN;
     struct Lds {
         uint32_t seen_cache[kSeenCache];
         int cand_id[kWave];
@@ -113,7 +136,7 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
     const int lane = threadIdx.x;
     float *okey = reinterpret_cast<float *>(lds.heap);
     int *oval = reinterpret_cast<int *>(okey + kHeapCells);
-    OpenList<H> open;
+    Open open;
     open.cells = lds.heap;
     int *cand_id = lds.cand_id;
     float *cand_key = lds.cand_key;
@@ -123,6 +146,8 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
     const bool use_cache = a.n_storage <= (0xffff << kSeenCacheLog2);
     const int deg = a.deg;
     uint32_t *seen = a.seen + (size_t)blockIdx.x * (size_t)a.slot_stride;
+    // after the visited slice and the result values (H of them, rounded up)
+    open.deep = reinterpret_cast<int2 *>(seen + a.words_per_slot + (H + kWave - 1) / kWave * kWave);
 
     for (;;) {
         int q = 0;
@@ -229,7 +254,7 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
             }
             return before;
         };
-        int v = load_row(OpenList<H>::rl(open.Av, 1));
+        int v = load_row(Open::rl(open.Av, 1));
         uint32_t before = test_and_set(v);
         for (int step = 0; step < a.max_iter; ++step) {
             int uk, u;
@@ -238,6 +263,7 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
             if (u == -1 || uk >= res.worst) break;
             n_expand += 1;
             int guess = -3, guess_row = -1;
+            bool popped = false;  // the pop has been finished
             if (u >= 0) {
                 n_adj += deg;
                 const bool fresh = !((before >> (v & 31)) & 1u);
@@ -251,14 +277,18 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
                     n_dist += n;
                     wave_sync();
                     PA_TIMER(3);
+                    // levels of the open list in device memory: their pair
+                    // was requested by the pop and has arrived with the rows
+                    open.pop_finish(lane);
+                    popped = true;
 
                     const int d = float_to_key(lane < n ? cand_key[lane] : INFINITY);
                     const int id = lane < n ? cand_id[lane] : -1;
                     // most likely next node; first candidate on ties, as the
                     // rise of an equal key stops below the older one
                     const int d_min = -wave_max_key(-d);
-                    guess = OpenList<H>::rl(open.Av, 1);
-                    if (d_min < OpenList<H>::rl(open.Ak, 1) && d_min < res.worst)
+                    guess = Open::rl(open.Av, 1);
+                    if (d_min < Open::rl(open.Ak, 1) && d_min < res.worst)
                         guess = __builtin_amdgcn_readlane(
                             id, __builtin_ctzll(__ballot(d == d_min)));
                     guess_row = load_row(guess);
@@ -273,7 +303,7 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
                         const int vj = __builtin_amdgcn_readlane(id, j);
                         int mine[S];
                         res.begin_insert(dj, vj, lane, mine);
-                        const typename OpenList<H>::Leaf leaf = open.walk_to_large_leaf();
+                        const typename Open::Leaf leaf = open.walk_to_large_leaf();
                         res.finish_insert(lane, mine);
                         open.replace_leaf(leaf, dj, vj, lane);
                         n_admit += 1;
@@ -281,7 +311,8 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
                     PA_TIMER(4);
                 }
             }
-            const int r = OpenList<H>::rl(open.Av, 1);
+            if (!popped) open.pop_finish(lane);
+            const int r = Open::rl(open.Av, 1);
             v = r == guess ? guess_row : load_row(r);
             before = test_and_set(v);
             PA_TIMER(1);
@@ -568,8 +599,10 @@ int make_plan(int64_t n_storage, int64_t batch, int dp, int ef_total, Plan *p) {
     if (slots < 1) slots = 1;
     p->n_slots = (int)slots;
     p->words_per_slot = round_up((n_storage + 31) / 32, kSlotAlignWords);
-    // a slot: the visited slice, then the values of the result list
-    p->slot_stride = p->words_per_slot + round_up(p->H, kWave);
+    // a slot: the visited slice, the values of the result list, the levels
+    // of the open list that are kept in device memory (8 bytes a cell)
+    p->slot_stride = p->words_per_slot + round_up(p->H, kWave) +
+                     round_up(2 * open_list_deep_cells(p->H, deep_from(p->H)), kWave);
     p->workspace_bytes =
         kWorkCounterBytes + (size_t)p->n_slots * p->slot_stride * 4;
     return PA_OK;
