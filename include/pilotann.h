@@ -237,6 +237,25 @@ int pa_traverse_refine(int64_t *out_I, float *out_D, int64_t *buf_I,
                        int n_init, int n_buffers, int k, int ef_search);
 
 /*
+ * Nearest-neighbour candidates for graph construction, the step the reference
+ * leaves to faiss (pilot_ann/utils/graphs.py:15-20,52-56; no entry point of
+ * the reference's extension corresponds to it).  For each of m query rows the
+ * `keep` (64 or 128) base rows with the smallest
+ * |x_j|^2 - 2 q_i . x_j, products in half precision with float accumulation,
+ * unordered.  query_f16 [m * d] and base_f16 [n * d] are IEEE half rows,
+ * base_norm [n] the squared lengths; d % 8 == 0; n >= 1.  The base rows are
+ * dealt to n_seg workgroups per 128 query rows (n_seg > 1 when m is too small
+ * to fill the device); segment s of query i leaves its list at
+ * cand_score / cand_id [(s * m + i) * pa_knn_list_capacity(keep)], of which
+ * the first cand_count [s * m + i] (at most keep) entries are valid.  Device
+ * pointers; enqueued on `stream`.
+ */
+int64_t pa_knn_list_capacity(int keep);
+int pa_knn(float *cand_score, int32_t *cand_id, int32_t *cand_count,
+           const void *query_f16, const void *base_f16, const float *base_norm,
+           int64_t m, int64_t n, int d, int keep, int n_seg, void *stream);
+
+/*
  * The reference's operator hooks (extension/ops_cpu.cpp:8-95,
  * pilot_ann/kernels/__init__.py:5-35): one call of a heap primitive of
  * extension/inc/heapq.cuh on a host array heap of n (key, value) cells, a set

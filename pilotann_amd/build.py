@@ -11,7 +11,7 @@ CSRC = os.path.join(HERE, 'csrc')
 LIB = os.path.join(CSRC, 'libpilotann.so')
 
 HIP_SOURCES = ['traverse.hip', 'refine.hip', 'route.hip', 'rotate.hip',
-               'pipeline.hip']
+               'knn.hip', 'pipeline.hip']
 CXX_SOURCES = ['host_search.cpp']
 
 HIP_FLAGS = [

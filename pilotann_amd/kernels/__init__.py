@@ -298,6 +298,71 @@ def entry_distances(query: torch.Tensor, entry_vectors: torch.Tensor):
     return distances
 
 
+# ---- nearest-neighbour candidates for the graph builder -----------------------
+
+class HalfRows:
+    """Rows prepared for :func:`knn_candidates`: a half-precision copy, scaled
+    into [-1, 1], padded with zeros to a multiple of 128 rows and 64 columns
+    (what the kernel reads without bounds checks), and the squared lengths of
+    the scaled rows."""
+
+    def __init__(self, rows: torch.Tensor, scale: float = None):
+        _check(rows, 'rows', 2, torch.float32, True)
+        n, d = rows.shape
+        if scale is None:
+            scale = 1.0 / max(float(rows.abs().max()), 1e-30) if n else 1.0
+        self.n, self.d, self.scale = n, d, scale
+        n_pad, d_pad = -(-max(n, 1) // 128) * 128, -(-d // 64) * 64
+        self.half = torch.zeros(n_pad, d_pad, dtype=torch.float16, device=rows.device)
+        self.half[:n, :d] = rows * scale
+        self.norm = torch.zeros(n_pad, dtype=torch.float32, device=rows.device)
+        self.norm[:n] = (rows * scale).square().sum(-1)
+
+
+def knn_candidates(query, base, keep: int, n_seg: int = None):
+    """For every row of ``query`` the ``keep`` (64 or 128) rows of ``base``
+    that are closest by half-precision products (``pa_knn``; the step the
+    reference leaves to faiss, ``pilot_ann/utils/graphs.py:15-20``).
+    ``query`` / ``base``: float32 device tensors or :class:`HalfRows` (pass the
+    same object for both to rank a set against itself).  Returns ids
+    ``[m, keep]`` (int64, ``-1`` where ``base`` has fewer rows) in no
+    particular order; rank them with exact distances."""
+    if not isinstance(base, HalfRows):
+        base = HalfRows(base)
+    if not isinstance(query, HalfRows):
+        query = HalfRows(query, scale=base.scale)
+    _require(query.d == base.d, 'query.size(-1) == base.size(-1)')
+    _require(query.half.device == base.half.device, 'query.device == base.device')
+    _require(base.n >= 1, 'base.size(0) >= 1')
+    m, n, device = query.n, base.n, base.half.device
+    if m == 0:
+        return torch.empty(0, keep, dtype=torch.long, device=device)
+    if n_seg is None:
+        # enough workgroups for two per compute unit
+        blocks, tiles = -(-m // 128), -(-n // 128)
+        n_seg = max(1, min(tiles, -(-512 // blocks)))
+    cap = int(_lib.lib().pa_knn_list_capacity(int(keep)))
+    _require(cap > 0, 'keep is 64 or 128')
+    score = torch.empty(n_seg, m, cap, dtype=torch.float32, device=device)
+    ids = torch.empty(n_seg, m, cap, dtype=torch.int32, device=device)
+    count = torch.empty(n_seg, m, dtype=torch.int32, device=device)
+    with torch.cuda.device(device):
+        _lib.check(_lib.lib().pa_knn(
+            _ptr(score), _ptr(ids), _ptr(count), _ptr(query.half), _ptr(base.half),
+            _ptr(base.norm), m, n, base.half.size(1), int(keep), n_seg, _stream()),
+            'pa_knn')
+    score, ids = score[:, :, :keep], ids[:, :, :keep]
+    valid = torch.arange(keep, device=device).view(1, 1, keep) < count.unsqueeze(-1)
+    ids = torch.where(valid, ids.long(), torch.full_like(ids, -1, dtype=torch.long))
+    if n_seg == 1:
+        return ids[0]
+    score = torch.where(valid, score, torch.full_like(score, float('inf')))
+    score = score.permute(1, 0, 2).reshape(m, n_seg * keep)
+    ids = ids.permute(1, 0, 2).reshape(m, n_seg * keep)
+    top = torch.topk(score, min(keep, score.size(1)), dim=-1, largest=False)
+    return torch.gather(ids, 1, top.indices)
+
+
 # ---- the reference's operator hooks ------------------------------------------
 
 def _heap(keys, values):

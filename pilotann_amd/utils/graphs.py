@@ -18,6 +18,10 @@ def knn_graph(x: torch.Tensor, k: int, chunk: int = None,
     a GPU) is used for the N×N products only."""
     n = x.size(0)
     k = min(k, n - 1)
+    # the kernel's candidates are ranked in half precision: 16 more than
+    # asked for are taken, so that float32 can settle the last places
+    if x.is_cuda and x.dtype == torch.float32 and 1 <= k <= 111 and n > 128:
+        return _knn_graph_device(x, k)
     if chunk is None:
         chunk = max(64, min(4096, (1 << 29) // max(n, 1)))
     norms = x.float().square().sum(-1)
@@ -39,6 +43,40 @@ def knn_graph(x: torch.Tensor, k: int, chunk: int = None,
         dists.append(top.values + norms[lo:lo + chunk].unsqueeze(-1))
         del d, dots
     return torch.cat(ids), torch.cat(dists).clamp_(min=0.0)
+
+
+def _knn_graph_device(x: torch.Tensor, k: int, rows_per_pass: int = None):
+    """:func:`knn_graph` on the device: candidates from the fused
+    half-precision kernel (``kernels.knn_candidates``, more of them than
+    asked for), then exact float32 distances to those candidates decide."""
+    from .. import kernels
+    n, d = x.shape
+    keep = 64 if k + 1 <= 48 else 128
+    rows = kernels.HalfRows(x)
+    out_i = torch.empty(n, k, dtype=torch.long, device=x.device)
+    out_d = torch.empty(n, k, dtype=torch.float32, device=x.device)
+    # candidate lists of a pass: 2 * (keep + 256) * 4 bytes a row
+    pass_rows = 1 << 21
+    if rows_per_pass is None:
+        rows_per_pass = max(256, min(8192, (1 << 29) // (keep * d)))
+    for lo in range(0, n, pass_rows):
+        hi = min(n, lo + pass_rows)
+        query = kernels.HalfRows.__new__(kernels.HalfRows)
+        query.n, query.d, query.scale = hi - lo, d, rows.scale
+        query.half, query.norm = rows.half[lo:], rows.norm[lo:]
+        cand = kernels.knn_candidates(query, rows, keep)
+        own = torch.arange(lo, hi, device=x.device).unsqueeze(-1)
+        for a in range(0, hi - lo, rows_per_pass):
+            b = min(hi - lo, a + rows_per_pass)
+            c = cand[a:b]
+            diff = x[c.clamp(min=0)] - x[lo + a:lo + b].unsqueeze(1)
+            d2 = diff.square_().sum(-1)
+            d2[(c < 0) | (c == own[a:b])] = float('inf')
+            top = torch.topk(d2, k, dim=-1, largest=False)
+            out_i[lo + a:lo + b] = torch.gather(c, 1, top.indices)
+            out_d[lo + a:lo + b] = top.values
+            del diff, d2
+    return out_i, out_d
 
 
 def _occlusion_prune(x, cand, cand_d, m_keep: int, fill: bool, chunk: int):

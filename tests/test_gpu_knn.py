@@ -1,0 +1,135 @@
+"""The fused nearest-neighbour kernel of the graph builder (`pa_knn`,
+`kernels.knn_candidates`, the device path of `utils.knn_graph`) against an
+exact float64 ranking.  The kernel ranks with half-precision products, so
+what is asserted is that the exact neighbours are among its candidates and
+that the builder's table, which ranks the candidates again in float32, is
+the exact one up to ties."""
+import ctypes
+
+import pytest
+import torch
+
+from pilotann_amd import _lib, kernels, utils
+from pilotann_amd.utils import graphs
+
+pytestmark = pytest.mark.gpu
+
+
+def exact_neighbours(query, base, k, exclude_self=False):
+    d = torch.cdist(query.double(), base.double())
+    if exclude_self:
+        d.fill_diagonal_(float('inf'))
+    return torch.topk(d, k, dim=-1, largest=False)
+
+
+def overlap(got, want):
+    hits = sum(len(set(a) & set(b)) for a, b in zip(got.tolist(), want.tolist()))
+    return hits / want.numel()
+
+
+@pytest.mark.parametrize('n,d,k', [
+    (129, 8, 5), (1000, 64, 10), (5000, 72, 47), (5000, 72, 48),
+    (20000, 96, 64), (3000, 200, 111), (3000, 200, 127), (12345, 768, 80),
+])
+def test_knn_table_is_the_exact_one(n, d, k, device):
+    print('knn case', n, d, k, flush=True)
+    x = utils.gaussian_mixture(n, d, 16, 1.0, seed=n + d, normalize=(d > 100),
+                               decay=0.5).to(device)
+    ids, d2 = utils.knn_graph(x, k)          # the kernel for n > 128 and k <= 111
+    torch.cuda.synchronize()
+    assert ids.shape == (n, k) and d2.shape == (n, k)
+    assert ids.dtype == torch.long and int(ids.min()) >= 0 and int(ids.max()) < n
+    assert not bool((ids == torch.arange(n, device=device).unsqueeze(-1)).any())
+    assert bool((d2[:, 1:] >= d2[:, :-1]).all())
+    rows = slice(0, min(n, 1500))
+    want = exact_neighbours(x[rows], x, k + 1)
+    # drop the row itself from the exact ranking (first place, distance 0)
+    keep = want.indices != torch.arange(rows.stop, device=device).unsqueeze(-1)
+    want_ids = want.indices[keep].view(rows.stop, k)
+    want_d = want.values[keep].view(rows.stop, k)
+    # the same distances place for place (ids may swap inside exact ties)
+    assert torch.allclose(d2[rows].double().sqrt(), want_d, rtol=1e-5, atol=1e-6)
+    assert overlap(ids[rows], want_ids) > 0.9999
+    # distances are those of the ids returned
+    back = (x[ids[:64]] - x[:64].unsqueeze(1)).square().sum(-1)
+    assert torch.allclose(back, d2[:64], rtol=1e-5, atol=1e-6)
+
+
+def test_the_device_table_agrees_with_the_host_path(device):
+    x = utils.gaussian_mixture(4000, 64, 8, 1.0, seed=5, decay=0.5)
+    host_ids, host_d = utils.knn_graph(x, 20)
+    dev_ids, dev_d = utils.knn_graph(x.to(device), 20)
+    assert torch.allclose(host_d, dev_d.cpu(), rtol=1e-4, atol=1e-5)
+    assert overlap(dev_ids.cpu(), host_ids) > 0.9995
+
+
+@pytest.mark.parametrize('m,n,d,keep', [
+    (1, 130, 64, 64), (300, 20000, 96, 128), (257, 4000, 128, 64), (1000, 1000, 40, 128),
+])
+def test_candidates_of_a_few_queries_over_segments(m, n, d, keep, device):
+    """Few query rows: the base rows are dealt to several workgroups per 128
+    queries and the lists merged; the exact nearest keep / 2 rows must be
+    among the keep candidates."""
+    print('knn candidates', m, n, d, keep, flush=True)
+    g = torch.Generator().manual_seed(m + n)
+    base = torch.randn(n, d, generator=g).to(device)
+    query = torch.randn(m, d, generator=g).to(device)
+    cand = kernels.knn_candidates(query, base, keep)
+    torch.cuda.synchronize()
+    assert cand.shape == (m, keep) and int(cand.max()) < n and int(cand.min()) >= 0
+    srt = torch.sort(cand, dim=1).values
+    assert bool((srt[:, 1:] != srt[:, :-1]).all())            # no id twice
+    want = exact_neighbours(query, base, keep // 2).indices
+    assert overlap(cand, want) > 0.9995
+    # one segment and many give the same sets when nothing is tied
+    one = kernels.knn_candidates(query, base, keep, n_seg=1)
+    many = kernels.knn_candidates(query, base, keep, n_seg=min(7, -(-n // 128)))
+    assert overlap(one, want) > 0.9995 and overlap(many, want) > 0.9995
+
+
+def test_fewer_base_rows_than_candidates(device):
+    base = torch.randn(50, 64, generator=torch.Generator().manual_seed(1)).to(device)
+    cand = kernels.knn_candidates(base, base, 64)
+    torch.cuda.synchronize()
+    assert cand.shape == (50, 64)
+    assert bool(((cand >= 0).sum(1) == 50).all())             # every row, once, then -1
+    assert bool((torch.sort(cand, 1).values[:, 14:] == torch.arange(50, device=device)).all())
+
+
+def test_repeated_rows_and_large_values(device):
+    """Rows that occur twice are each other's nearest neighbour at distance
+    zero (only the row itself is dropped); values far outside the half
+    range are scaled before the conversion."""
+    g = torch.Generator().manual_seed(3)
+    x = 1e6 * torch.randn(2000, 64, generator=g)
+    x[1000:1100] = x[:100]
+    ids, d2 = utils.knn_graph(x.to(device), 8)
+    assert bool((ids[:100, 0].cpu() == torch.arange(1000, 1100)).all())
+    assert bool((d2[:100, 0] == 0).all())
+    # differences first: the product form of cdist cancels at this scale
+    exact = (x[:300].double().unsqueeze(1) - x.double().unsqueeze(0)).square().sum(-1)
+    exact[torch.arange(300), torch.arange(300)] = float('inf')
+    want = torch.topk(exact, 8, dim=-1, largest=False).values
+    assert torch.allclose(d2[:300].cpu().double(), want, rtol=1e-5)
+
+
+def test_knn_argument_errors(device):
+    lib = _lib.lib()
+    buf = torch.zeros(1 << 16, device=device)
+    p = ctypes.c_void_p(buf.data_ptr())
+    none = ctypes.c_void_p(None)
+    def call(m=128, n=128, d=64, keep=64, n_seg=1, q=p):
+        return lib.pa_knn(p, p, p, q, p, p, m, n, d, keep, n_seg, none)
+    assert call(d=72) == lib.pa_knn(p, p, p, p, p, p, 128, 128, 8, 64, 1, none) != 0   # d % 64
+    assert call(keep=100) != 0
+    assert call(n=0) != 0
+    assert call(n_seg=0) != 0
+    assert call(m=-1) != 0
+    assert call(q=none) != 0
+    assert call(m=0) == 0
+    assert lib.pa_knn_list_capacity(64) == 320 and lib.pa_knn_list_capacity(128) == 384
+    with pytest.raises(RuntimeError):
+        kernels.knn_candidates(torch.zeros(4, 64), torch.zeros(200, 64, device=device), 64)
+    with pytest.raises(RuntimeError):
+        kernels.knn_candidates(torch.zeros(4, 32, device=device),
+                               torch.zeros(200, 64, device=device), 64)
