@@ -536,6 +536,10 @@ def main():
                          '(c5): write the stage\'s inputs to FILE after the '
                          'build, or read them from FILE if it exists (for '
                          'counter runs, which slow the build down)')
+    ap.add_argument('--knn-only', action='store_true',
+                    help="only time the graph builder's nearest-neighbour "
+                         "kernel (pa_knn) on the configuration's base set "
+                         "against itself, print its rate and exit")
     ap.add_argument('--copy-calibration', action='store_true',
                     help='only run a plain 1 GiB device copy five times (to '
                          'scale the FETCH_SIZE / WRITE_SIZE counters) and exit')
@@ -558,6 +562,11 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({'copy_calibration': '5 copies of 1 GiB (read 1 GiB, '
                                               'write 1 GiB each)'}))
+        return
+
+    if args.knn_only:
+        print(json.dumps(knn_figures(dict(CONFIGS[args.config], name=args.config),
+                                     args, 'cuda:0')), flush=True)
         return
 
     cfg = dict(CONFIGS[args.config], name=args.config)
@@ -737,6 +746,44 @@ def context_figures(line, args, cfg, index, stage, query, target, ef,
 
     if args.config == 'c3' and cfg['decay'] > 0 and not args.n_base:
         line['config']['isotropic_mixture'] = isotropic_twin(cfg, device, args)
+
+
+def knn_figures(cfg, args, device):
+    """The nearest-neighbour kernel of the graph builder on the rotated base
+    set against itself (what `graph_init` runs first): seconds per pass and
+    the rate of its half-precision products against the dense fp16 MFMA
+    peak."""
+    from pilotann_amd import kernels, utils
+    torch.cuda.set_device(0)
+    if args.n_base:
+        cfg['n'] = args.n_base
+    x, _, _ = make_data(dict(cfg, queries=8), device)
+    x, _ = utils.svd(x, max_size=10_000_000, seed=cfg['seed'])
+    rows = kernels.HalfRows(x)
+    n, d = x.shape
+    times = []
+    for _ in range(max(2, args.warmup)):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        cand = kernels.knn_candidates(rows, rows, 128)
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+    t0 = time.perf_counter()
+    ids, _ = utils.knn_graph(x, 80)
+    torch.cuda.synchronize()
+    whole = time.perf_counter() - t0
+    flops = 2.0 * n * n * rows.half.size(1)
+    return {
+        'kernel': 'knn_kernel<128>', 'rows': n, 'd': d,
+        'seconds_per_pass': round(min(times), 3),
+        'roofline': {'bound': 'mfma', 'achieved': round(flops / min(times) / 1e12, 1),
+                     'peak': 2500.0, 'unit': 'TFLOP/s',
+                     'frac': round(flops / min(times) / 2.5e15, 4)},
+        'knn_graph_seconds': round(whole, 2),
+        'what': 'kernels.knn_candidates(x, x, 128): the 128 closest rows of every '
+                'row by fp16 products; knn_graph adds the exact float32 ranking '
+                'of those candidates (80 kept)',
+    }
 
 
 def isotropic_twin(cfg, device, args):
