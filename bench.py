@@ -466,6 +466,8 @@ def cpu_full_graph_baseline(index, query, stage, target, k, budget_s=6.0):
         t, out_I = run(n_sample, ef_search)
         rec = utils.recall(out_I, target[:n_sample])
         sweep.append(dict(ef_search=ef_search, recall=round(rec, 4)))
+        log(f'[bench] host search alone: ef_search={ef_search} recall@{k}={rec:.4f} '
+            f'({n_sample} queries in {t:.2f}s)')
         if rec >= 0.90:
             chosen = ef_search
             break
@@ -536,6 +538,11 @@ def main():
                          '(c5): write the stage\'s inputs to FILE after the '
                          'build, or read them from FILE if it exists (for '
                          'counter runs, which slow the build down)')
+    ap.add_argument('--full-index', action='store_true',
+                    help='configurations that build the device stage only '
+                         '(c5): build the whole index instead (full graph of '
+                         'all nodes, the reference\'s sampler, host and device '
+                         'refine), which takes minutes')
     ap.add_argument('--knn-only', action='store_true',
                     help="only time the graph builder's nearest-neighbour "
                          "kernel (pa_knn) on the configuration's base set "
@@ -578,6 +585,10 @@ def main():
         cfg['decay'] = args.decay
     device = 'cuda:0'
     torch.cuda.set_device(0)
+    if args.full_index:
+        cfg['stage_only'] = False
+        from pilotann_amd.utils import graphs
+        graphs.progress = lambda text: log('[bench] ' + text)
     if args.stage_cache and not cfg.get('stage_only'):
         ap.error('--stage-cache is for configurations that build the device '
                  'stage only')

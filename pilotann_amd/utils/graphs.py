@@ -1,14 +1,23 @@
-"""Proximity graphs in the reference's layout, built with torch only.
+"""Proximity graphs in the reference's layout.
 
 Layout (``pilot_ann/utils/graphs.py:22-40``): ``indptr[i] = i * n_neighbors``,
 ``indices`` padded with ``-1`` after a row's last neighbour.  A subgraph keeps
 global ids and one (possibly empty) row per global node
 (``graphs.py:118-129``).  Construction differs from the reference, which
-delegates to faiss: here an exact k-nearest-neighbour table is pruned with the
-usual occlusion rule and completed with reverse edges.  Everything runs on the
-device ``x`` lives on, so a million-node build is a matter of a GPU minute.
+delegates to faiss: here an exact k-nearest-neighbour table (on a GPU: the
+fused half-precision kernel ``pa_knn`` plus an exact float32 ranking of its
+candidates) is pruned with the usual occlusion rule and completed with
+reverse edges.  Everything runs on the device ``x`` lives on: a million
+768-dimensional nodes take ten seconds on an MI355X, ten million five and a
+half minutes.
 """
 import torch
+
+
+# Called with a short text when a long step of a build has finished a part
+# (a pass of the neighbour kernel over two million rows, say): a caller that
+# must show signs of life sets it (``graphs.progress = print``).
+progress = None
 
 
 def knn_graph(x: torch.Tensor, k: int, chunk: int = None,
@@ -76,6 +85,8 @@ def _knn_graph_device(x: torch.Tensor, k: int, rows_per_pass: int = None):
             out_i[lo + a:lo + b] = torch.gather(c, 1, top.indices)
             out_d[lo + a:lo + b] = top.values
             del diff, d2
+        if progress is not None:
+            progress(f'neighbour table: {hi} of {n} rows')
     return out_i, out_d
 
 
