@@ -45,8 +45,8 @@ CONFIGS = {
     'c3': dict(n=1_000_000, d=768, dp=128, n_centers=1024, sigma=1.0,
                decay=0.5, normalize=True, ratio=0.25, graph='nsw64',
                entry='router64x64', queries=10_000, k=10,
-               ef_sweep=[4, 8, 16, 24, 32, 48, 64], seed=301,
-               curve=[32, 48, 64, 96, 128, 192, 256]),
+               ef_sweep=[4, 6, 8, 12, 16, 24, 32, 48, 64], seed=301,
+               curve=[4, 6, 8, 16, 32, 64, 128, 256]),
     # large result lists: top-100, ef 256 / 512 (heaps of 1024 / 2048 entries)
     'c4': dict(n=1_000_000, d=768, dp=128, n_centers=1024, sigma=1.0,
                decay=0.5, normalize=True, ratio=0.5, graph='nsw64',
@@ -56,7 +56,7 @@ CONFIGS = {
     'c2': dict(n=1_000_000, d=96, dp=64, n_centers=256, sigma=1.0,
                decay=0.5, normalize=False, ratio=0.25, graph='nsw32',
                entry='router32x32', queries=10_000, k=10,
-               ef_sweep=[8, 16, 32, 64, 128], seed=201),
+               ef_sweep=[4, 6, 8, 16, 32, 64, 128], seed=201),
     # the memory-bounded case: 10M x 768, 2.5M reduced rows and their graph
     # on the device.  Only the device stage is built: the subgraph on a seeded
     # random quarter of the nodes (the reference's sampler walks the full

@@ -240,7 +240,7 @@ int pa_traverse_refine(int64_t *out_I, float *out_D, int64_t *buf_I,
  * Nearest-neighbour candidates for graph construction, the step the reference
  * leaves to faiss (pilot_ann/utils/graphs.py:15-20,52-56; no entry point of
  * the reference's extension corresponds to it).  For each of m query rows the
- * `keep` (64 or 128) base rows with the smallest
+ * `keep` (64, 128, 256 or 512) base rows with the smallest
  * |x_j|^2 - 2 q_i . x_j, products in half precision with float accumulation,
  * unordered.  query_f16 [m * d] and base_f16 [n * d] are IEEE half rows,
  * base_norm [n] the squared lengths; d % 8 == 0; n >= 1.  The base rows are
@@ -254,6 +254,20 @@ int64_t pa_knn_list_capacity(int keep);
 int pa_knn(float *cand_score, int32_t *cand_id, int32_t *cand_count,
            const void *query_f16, const void *base_f16, const float *base_norm,
            int64_t m, int64_t n, int d, int keep, int n_seg, void *stream);
+
+/*
+ * Occlusion pruning of candidate lists, the edge selection of the graph
+ * builder (faiss' part in the reference, pilot_ann/utils/graphs.py:15-20,52-56;
+ * no entry point of the reference's extension corresponds to it).  For each of
+ * n nodes: cand_dist [n * k] are the distances of its k <= 512 candidates,
+ * closest first, pair [n * k * k] the distances between its candidates.
+ * Candidate j is kept unless an earlier kept candidate r has
+ * pair[j][r] < cand_dist[j]; selected [n * m_keep] receives the positions of
+ * the kept candidates in order, then (with fill != 0) the closest rejected
+ * ones, then -1.  Device pointers; enqueued on `stream`.
+ */
+int pa_graph_prune(int32_t *selected, const float *pair, const float *cand_dist,
+                   int64_t n, int k, int m_keep, int fill, void *stream);
 
 /*
  * The reference's operator hooks (extension/ops_cpu.cpp:8-95,

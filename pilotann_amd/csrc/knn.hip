@@ -258,9 +258,63 @@ __global__ __launch_bounds__(256) void knn_kernel(KnnArgs a) {
     if (t < kBM && q0 + t < a.m) a.cand_count[(size_t)seg * a.m + q0 + t] = count[t];
 }
 
+// Occlusion pruning of a node's candidate list (closest first): candidate j
+// is kept unless a candidate kept before it is closer to it than the node
+// itself is, until m_keep are kept; with `fill` the closest rejected ones top
+// the row up to m_keep.  One wavefront per node; the kept set is a bit mask
+// that every lane carries, a step tests one row of the node's table of
+// candidate-to-candidate distances against it.
+__global__ __launch_bounds__(256) void prune_kernel(
+    const float *__restrict__ pair, const float *__restrict__ cand_dist,
+    int32_t *__restrict__ selected, int64_t n, int k, int m_keep, int fill) {
+    constexpr int kWords = 8;  // k <= 512
+    const int lane = threadIdx.x & (kWave - 1);
+    const int64_t node = (int64_t)blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
+    if (node >= n) return;
+    const float *table = pair + (size_t)node * k * k;
+    const float *dist = cand_dist + (size_t)node * k;
+    int32_t *out = selected + (size_t)node * m_keep;
+    unsigned long long kept[kWords];
+#pragma unroll
+    for (int w = 0; w < kWords; ++w) kept[w] = 0;
+    int count = 0;
+    for (int j = 0; j < k && count < m_keep; ++j) {
+        const float own = dist[j];
+        bool hit = false;
+        // only candidates before j can have been kept
+#pragma unroll
+        for (int w = 0; w < kWords; ++w) {
+            const int r = 64 * w + lane;
+            if (64 * w < j && r < j && ((kept[w] >> lane) & 1ull))
+                hit |= table[(size_t)j * k + r] < own;
+        }
+        if (!__ballot(hit)) {
+#pragma unroll
+            for (int w = 0; w < kWords; ++w)
+                if (j >> 6 == w) kept[w] |= 1ull << (j & 63);
+            if (lane == 0) out[count] = j;
+            count += 1;
+        }
+    }
+    if (fill) {
+        for (int j = 0; j < k && count < m_keep; ++j) {
+            bool is_kept = false;
+#pragma unroll
+            for (int w = 0; w < kWords; ++w)
+                if (j >> 6 == w) is_kept = (kept[w] >> (j & 63)) & 1ull;
+            if (is_kept) continue;
+            if (lane == 0) out[count] = j;
+            count += 1;
+        }
+    }
+    for (int i = count + lane; i < m_keep; i += kWave) out[i] = -1;
+}
+
 }  // namespace
 
-extern "C" int64_t pa_knn_list_capacity(int keep) { return keep + kSlack + kBN; }
+extern "C" int64_t pa_knn_list_capacity(int keep) {
+    return keep == 64 || keep == 128 || keep == 256 || keep == 512 ? keep + kSlack + kBN : 0;
+}
 
 extern "C" int pa_knn(float *cand_score, int32_t *cand_id, int32_t *cand_count,
                       const void *query_f16, const void *base_f16,
@@ -269,7 +323,7 @@ extern "C" int pa_knn(float *cand_score, int32_t *cand_id, int32_t *cand_count,
     if (m < 0 || n < 0 || n_seg < 1 || n_seg > 65535) return PA_E_SHAPE;
     if (n >= (1ll << 31) || (m + kBM - 1) / kBM >= (1ll << 31)) return PA_E_RANGE;
     if (d <= 0 || d % kChunk) return PA_E_DIM;
-    if (keep != 64 && keep != 128) return PA_E_SHAPE;
+    if (keep != 64 && keep != 128 && keep != 256 && keep != 512) return PA_E_SHAPE;
     if (m == 0) return PA_OK;
     if (n == 0) return PA_E_SHAPE;
     if (!cand_score || !cand_id || !cand_count || !query_f16 || !base_f16 || !base_norm)
@@ -282,9 +336,23 @@ extern "C" int pa_knn(float *cand_score, int32_t *cand_id, int32_t *cand_count,
     a.m = m, a.n = n, a.d = d, a.n_seg = n_seg;
     const dim3 grid((unsigned)((m + kBM - 1) / kBM), (unsigned)n_seg);
     hipStream_t stream = (hipStream_t)stream_;
-    if (keep == 64)
-        knn_kernel<64><<<grid, 256, 0, stream>>>(a);
-    else
-        knn_kernel<128><<<grid, 256, 0, stream>>>(a);
+    switch (keep) {
+        case 64: knn_kernel<64><<<grid, 256, 0, stream>>>(a); break;
+        case 128: knn_kernel<128><<<grid, 256, 0, stream>>>(a); break;
+        case 256: knn_kernel<256><<<grid, 256, 0, stream>>>(a); break;
+        default: knn_kernel<512><<<grid, 256, 0, stream>>>(a);
+    }
+    return (int)hipGetLastError();
+}
+
+extern "C" int pa_graph_prune(int32_t *selected, const float *pair,
+                              const float *cand_dist, int64_t n, int k,
+                              int m_keep, int fill, void *stream_) {
+    if (n < 0 || k < 1 || k > 512 || m_keep < 1) return PA_E_SHAPE;
+    if ((n + 3) / 4 >= (1ll << 31)) return PA_E_RANGE;
+    if (n == 0) return PA_OK;
+    if (!selected || !pair || !cand_dist) return PA_E_NULL;
+    prune_kernel<<<(unsigned)((n + 3) / 4), 256, 0, (hipStream_t)stream_>>>(
+        pair, cand_dist, selected, n, k, m_keep, fill);
     return (int)hipGetLastError();
 }

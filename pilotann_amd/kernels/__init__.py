@@ -320,7 +320,7 @@ class HalfRows:
 
 
 def knn_candidates(query, base, keep: int, n_seg: int = None):
-    """For every row of ``query`` the ``keep`` (64 or 128) rows of ``base``
+    """For every row of ``query`` the ``keep`` (64, 128, 256 or 512) rows of ``base``
     that are closest by half-precision products (``pa_knn``; the step the
     reference leaves to faiss, ``pilot_ann/utils/graphs.py:15-20``).
     ``query`` / ``base``: float32 device tensors or :class:`HalfRows` (pass the
@@ -342,7 +342,7 @@ def knn_candidates(query, base, keep: int, n_seg: int = None):
         blocks, tiles = -(-m // 128), -(-n // 128)
         n_seg = max(1, min(tiles, -(-512 // blocks)))
     cap = int(_lib.lib().pa_knn_list_capacity(int(keep)))
-    _require(cap > 0, 'keep is 64 or 128')
+    _require(cap > 0, 'keep is 64, 128, 256 or 512')
     score = torch.empty(n_seg, m, cap, dtype=torch.float32, device=device)
     ids = torch.empty(n_seg, m, cap, dtype=torch.int32, device=device)
     count = torch.empty(n_seg, m, dtype=torch.int32, device=device)
@@ -361,6 +361,24 @@ def knn_candidates(query, base, keep: int, n_seg: int = None):
     ids = ids.permute(1, 0, 2).reshape(m, n_seg * keep)
     top = torch.topk(score, min(keep, score.size(1)), dim=-1, largest=False)
     return torch.gather(ids, 1, top.indices)
+
+
+def graph_prune(pair: torch.Tensor, cand_dist: torch.Tensor, m_keep: int, fill: bool):
+    """Occlusion pruning of candidate lists (``pa_graph_prune``): ``pair``
+    ``[n, k, k]`` distances between a node's candidates, ``cand_dist``
+    ``[n, k]`` their distances to the node, closest first.  Returns the
+    positions ``[n, m_keep]`` (int64, ``-1`` padded) of the candidates kept, in
+    order, topped up with the closest rejected ones when ``fill``."""
+    _check(pair, 'pair', 3, torch.float32, True)
+    _check(cand_dist, 'cand_dist', 2, torch.float32, True)
+    n, k = cand_dist.shape
+    _require(pair.shape == (n, k, k), 'pair.shape == (n, k, k)')
+    selected = torch.empty(n, int(m_keep), dtype=torch.int32, device=pair.device)
+    with torch.cuda.device(pair.device):
+        _lib.check(_lib.lib().pa_graph_prune(
+            _ptr(selected), _ptr(pair), _ptr(cand_dist), n, k, int(m_keep),
+            int(bool(fill)), _stream()), 'pa_graph_prune')
+    return selected.long()
 
 
 # ---- the reference's operator hooks ------------------------------------------

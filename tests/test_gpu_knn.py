@@ -30,12 +30,13 @@ def overlap(got, want):
 @pytest.mark.parametrize('n,d,k', [
     (129, 8, 5), (1000, 64, 10), (5000, 72, 47), (5000, 72, 48),
     (20000, 96, 64), (3000, 200, 111), (3000, 200, 127), (12345, 768, 80),
+    (9000, 64, 240), (3000, 128, 495), (3000, 128, 496),
 ])
 def test_knn_table_is_the_exact_one(n, d, k, device):
     print('knn case', n, d, k, flush=True)
     x = utils.gaussian_mixture(n, d, 16, 1.0, seed=n + d, normalize=(d > 100),
                                decay=0.5).to(device)
-    ids, d2 = utils.knn_graph(x, k)          # the kernel for n > 128 and k <= 111
+    ids, d2 = utils.knn_graph(x, k)          # the kernel for n > 128 and k <= 495
     torch.cuda.synchronize()
     assert ids.shape == (n, k) and d2.shape == (n, k)
     assert ids.dtype == torch.long and int(ids.min()) >= 0 and int(ids.max()) < n
@@ -65,6 +66,7 @@ def test_the_device_table_agrees_with_the_host_path(device):
 
 @pytest.mark.parametrize('m,n,d,keep', [
     (1, 130, 64, 64), (300, 20000, 96, 128), (257, 4000, 128, 64), (1000, 1000, 40, 128),
+    (200, 9000, 64, 256), (130, 5000, 96, 512),
 ])
 def test_candidates_of_a_few_queries_over_segments(m, n, d, keep, device):
     """Few query rows: the base rows are dealt to several workgroups per 128
@@ -128,8 +130,43 @@ def test_knn_argument_errors(device):
     assert call(q=none) != 0
     assert call(m=0) == 0
     assert lib.pa_knn_list_capacity(64) == 320 and lib.pa_knn_list_capacity(128) == 384
+    assert lib.pa_knn_list_capacity(512) == 768 and lib.pa_knn_list_capacity(100) == 0
     with pytest.raises(RuntimeError):
         kernels.knn_candidates(torch.zeros(4, 64), torch.zeros(200, 64, device=device), 64)
     with pytest.raises(RuntimeError):
         kernels.knn_candidates(torch.zeros(4, 32, device=device),
                                torch.zeros(200, 64, device=device), 64)
+
+
+@pytest.mark.parametrize('n,k,m_keep,fill', [
+    (1, 5, 3, True), (300, 64, 32, True), (300, 64, 32, False), (257, 240, 32, True),
+    (100, 512, 48, False), (50, 20, 32, True), (64, 130, 64, False),
+])
+def test_occlusion_pruning_equals_the_step_by_step_rule(n, k, m_keep, fill, device):
+    """`pa_graph_prune` against the rule written out on the host: candidates
+    closest first; one is kept unless an earlier kept one is closer to it
+    than the node is; `fill` tops up with the closest rejected ones."""
+    print('prune case', n, k, m_keep, fill, flush=True)
+    g = torch.Generator().manual_seed(n + k)
+    pts = torch.randn(n, k, 6, generator=g)
+    node = torch.randn(n, 1, 6, generator=g) * 0.3
+    d = (pts - node).square().sum(-1)
+    order = torch.argsort(d, dim=-1)
+    pts = torch.gather(pts, 1, order.unsqueeze(-1).expand(-1, -1, 6))
+    d = torch.gather(d, 1, order)
+    pair = (pts.unsqueeze(2) - pts.unsqueeze(1)).square().sum(-1).contiguous()
+    got = kernels.graph_prune(pair.to(device), d.contiguous().to(device), m_keep, fill).cpu()
+    want = torch.full((n, m_keep), -1, dtype=torch.long)
+    for i in range(n):
+        kept, rejected = [], []
+        for j in range(k):
+            if len(kept) < m_keep and not any(pair[i, j, r] < d[i, j] for r in kept):
+                kept.append(j)
+            else:
+                rejected.append(j)
+        row = kept + (rejected if fill else [])
+        row = row[:m_keep]
+        want[i, :len(row)] = torch.tensor(row, dtype=torch.long)
+    assert torch.equal(got, want)
+    with pytest.raises(RuntimeError):
+        kernels.graph_prune(pair[:, :, :-1].contiguous().to(device), d.to(device), m_keep, fill)
