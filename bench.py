@@ -290,6 +290,12 @@ def algorithmic_bytes(counters, B, dp, n_init):
             + C * (w + 4 * dp) + R * (w + 4))
 
 
+def traffic_key(cfg, B, ef):
+    """Name of a measured workload in profiles/traffic.json."""
+    return (f'{cfg["name"]}/n={cfg["n"]}/queries={B}/ef={ef}'
+            f'/spectrum_exponent={cfg["decay"]}')
+
+
 def measured_traffic(key, sources=TRAVERSAL_SOURCES):
     """Bytes per launch that left the L2 towards the fabric, from the
     rocprofv3 counter runs summarised under profiles/ (FETCH_SIZE and
@@ -631,7 +637,7 @@ def main():
     t = time_stage(stage, ef, args.steps, args.warmup)
     out_I, out_D = t['out_I'], t['out_D']
     launch_bytes, ms_per_step = t['launch_bytes'], t['ms_per_step']
-    key = f'{args.config}/n={cfg["n"]}/queries={B}/ef={ef}'
+    key = traffic_key(cfg, B, ef)
 
     line = {
         'metric': METRIC,
@@ -670,7 +676,7 @@ def main():
             if e not in recalls:
                 recalls[e] = round(end_to_end_recall(index, stage, e, target, k)[0], 4)
             o = time_stage(stage, e, max(3, args.steps // 2), 1)
-            rec = stage_record(o, B, f'{args.config}/n={cfg["n"]}/queries={B}/ef={e}')
+            rec = stage_record(o, B, traffic_key(cfg, B, e))
             line['config']['other_ef'].append(dict(
                 ef=e, recall_at_k=recalls[e],
                 queries_per_s=round(B / (o['ms_per_step'] * 1e-3), 1),
@@ -887,7 +893,7 @@ def device_refine_figures(cfg, index, stage, query, target, ef, host_top=None,
                  counters.cpu().tolist()))
     n_cand = cand_I.size(1)
     refine_traffic = measured_traffic(
-        f'{cfg["name"]}/n={cfg["n"]}/queries={B}/ef={ef}/refine',
+        traffic_key(cfg, B, ef) + '/refine',
         ('refine.hip', 'search_lists.h', 'device_common.h'))
     # query + candidates read + completed tails + adjacency ids + full rows
     # (4-byte id each) + buffer and top-k written

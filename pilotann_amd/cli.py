@@ -17,7 +17,7 @@ Datasets: the reference's names (``deep-1m``, ``text2img-10m``, ``wiki-1m``,
 ``--data_root``, default ``.dataset`` as in the reference), or a synthetic
 unit-norm Gaussian mixture, ``synth:<n>x<d>[:<centres>[:<spectrum
 exponent>]]``; the default is the shape of the headline benchmark
-(``synth:1000000x768:1024:0.5`` with ``--d_principle 128 --n_neighbors 64
+(``synth:1000000x768:1024:0`` with ``--d_principle 128 --n_neighbors 64
 --router router64x64``).
 
     python -m pilotann_amd.cli --dataset synth:200000x128:64:0.5 \\
@@ -41,7 +41,7 @@ def parse_dataset(name: str):
     parts = name[len('synth:'):].split(':')
     n, d = (int(v) for v in parts[0].lower().split('x'))
     centres = int(parts[1]) if len(parts) > 1 else 64
-    decay = float(parts[2]) if len(parts) > 2 else 0.5
+    decay = float(parts[2]) if len(parts) > 2 else 0.0
     return dict(n=n, d=d, n_centers=centres, sigma=1.0, decay=decay,
                 normalize=True, seed=7)
 
@@ -159,7 +159,7 @@ def main(argv=None):
                         choices=['hnsw', 'nsg'])
     parser.add_argument('--router', type=str, default='router64x64')
     parser.add_argument('--dataset', type=str,
-                        default='synth:1000000x768:1024:0.5')
+                        default='synth:1000000x768:1024:0')
     parser.add_argument('--data_root', default='.dataset',
                         help="directory of the reference's dataset folders")
     parser.add_argument('--refine', choices=['host', 'device'], default='host',

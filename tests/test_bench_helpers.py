@@ -48,7 +48,9 @@ def test_traffic_figures_name_the_sources_they_were_measured_with():
     assert len(bench.kernel_sources_sha16()) == 16
     for key, entry in entries.items():
         assert entry['hbm_bytes_per_launch'] > 0 and len(entry['kernel_sources_sha16']) == 16
-    value, fresh = bench.measured_traffic('c3/n=1000000/queries=10000/ef=64')
-    assert value == entries['c3/n=1000000/queries=10000/ef=64']['hbm_bytes_per_launch']
+    value, fresh = bench.measured_traffic('c3/n=1000000/queries=10000/ef=32/spectrum_exponent=0.0')
+    assert value == entries['c3/n=1000000/queries=10000/ef=32/spectrum_exponent=0.0']['hbm_bytes_per_launch']
     assert fresh in (True, False)
     assert bench.measured_traffic('no such workload') == (None, None)
+    cfg = dict(bench.CONFIGS['c3'], name='c3')
+    assert bench.traffic_key(cfg, 10000, 32) in entries
