@@ -242,8 +242,12 @@ int pa_traverse_refine(int64_t *out_I, float *out_D, int64_t *buf_I,
  * the reference's extension corresponds to it).  For each of m query rows the
  * `keep` (64, 128, 256 or 512) base rows with the smallest
  * |x_j|^2 - 2 q_i . x_j, products in half precision with float accumulation,
- * unordered.  query_f16 [m * d] and base_f16 [n * d] are IEEE half rows,
- * base_norm [n] the squared lengths; d % 8 == 0; n >= 1.  The base rows are
+ * unordered.  query_f16 and base_f16 hold m and n IEEE half rows of d
+ * elements, d % 64 == 0 (pad rows with zeros), and must be readable up to the
+ * next multiple of 128 rows (the kernel loads whole tiles; what the padding
+ * rows hold does not matter); base_norm [n] are the squared lengths of the
+ * base rows; n >= 1, and pa_knn_list_capacity() is 0 for any other `keep`.
+ * Values must fit the half range: scale both sets by one factor first.  The base rows are
  * dealt to n_seg workgroups per 128 query rows (n_seg > 1 when m is too small
  * to fill the device); segment s of query i leaves its list at
  * cand_score / cand_id [(s * m + i) * pa_knn_list_capacity(keep)], of which

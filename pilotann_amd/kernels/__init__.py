@@ -318,6 +318,15 @@ class HalfRows:
         self.norm = torch.zeros(n_pad, dtype=torch.float32, device=rows.device)
         self.norm[:n] = (rows * scale).square().sum(-1)
 
+    def rows(self, lo: int, hi: int) -> 'HalfRows':
+        """Rows ``lo .. hi`` as a set of their own (a view; ``lo`` a multiple
+        of 128, so that the padding still reaches a whole tile)."""
+        _require(lo % 128 == 0 and 0 <= lo < hi <= self.n, 'lo % 128 == 0, lo < hi <= n')
+        part = HalfRows.__new__(HalfRows)
+        part.n, part.d, part.scale = hi - lo, self.d, self.scale
+        part.half, part.norm = self.half[lo:], self.norm[lo:]
+        return part
+
 
 def knn_candidates(query, base, keep: int, n_seg: int = None):
     """For every row of ``query`` the ``keep`` (64, 128, 256 or 512) rows of ``base``

@@ -70,10 +70,7 @@ def _knn_graph_device(x: torch.Tensor, k: int, rows_per_pass: int = None):
         rows_per_pass = max(256, min(8192, (1 << 29) // (keep * d)))
     for lo in range(0, n, pass_rows):
         hi = min(n, lo + pass_rows)
-        query = kernels.HalfRows.__new__(kernels.HalfRows)
-        query.n, query.d, query.scale = hi - lo, d, rows.scale
-        query.half, query.norm = rows.half[lo:], rows.norm[lo:]
-        cand = kernels.knn_candidates(query, rows, keep)
+        cand = kernels.knn_candidates(rows.rows(lo, hi), rows, keep)
         own = torch.arange(lo, hi, device=x.device).unsqueeze(-1)
         for a in range(0, hi - lo, rows_per_pass):
             b = min(hi - lo, a + rows_per_pass)
