@@ -29,7 +29,7 @@ def knn_graph(x: torch.Tensor, k: int, chunk: int = None,
     k = min(k, n - 1)
     # the kernel's candidates are ranked in half precision: 16 more than
     # asked for are taken, so that float32 can settle the last places
-    if x.is_cuda and x.dtype == torch.float32 and 1 <= k <= 495 and n > 128:
+    if x.is_cuda and x.dtype == torch.float32 and 1 <= k <= 496 and n > 128:
         return _knn_graph_device(x, k)
     if chunk is None:
         chunk = max(64, min(4096, (1 << 29) // max(n, 1)))
@@ -60,7 +60,7 @@ def _knn_graph_device(x: torch.Tensor, k: int, rows_per_pass: int = None):
     asked for), then exact float32 distances to those candidates decide."""
     from .. import kernels
     n, d = x.shape
-    keep = next(size for size in (64, 128, 256, 512) if k + 17 <= size)
+    keep = next(size for size in (64, 128, 256, 512) if k + 16 <= size)
     rows = kernels.HalfRows(x)
     out_i = torch.empty(n, k, dtype=torch.long, device=x.device)
     out_d = torch.empty(n, k, dtype=torch.float32, device=x.device)

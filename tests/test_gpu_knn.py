@@ -30,13 +30,13 @@ def overlap(got, want):
 @pytest.mark.parametrize('n,d,k', [
     (129, 8, 5), (1000, 64, 10), (5000, 72, 47), (5000, 72, 48),
     (20000, 96, 64), (3000, 200, 111), (3000, 200, 127), (12345, 768, 80),
-    (9000, 64, 240), (3000, 128, 495), (3000, 128, 496),
+    (9000, 64, 240), (3000, 128, 496), (3000, 128, 497),
 ])
 def test_knn_table_is_the_exact_one(n, d, k, device):
     print('knn case', n, d, k, flush=True)
     x = utils.gaussian_mixture(n, d, 16, 1.0, seed=n + d, normalize=(d > 100),
                                decay=0.5).to(device)
-    ids, d2 = utils.knn_graph(x, k)          # the kernel for n > 128 and k <= 495
+    ids, d2 = utils.knn_graph(x, k)          # the kernel for n > 128 and k <= 496
     torch.cuda.synchronize()
     assert ids.shape == (n, k) and d2.shape == (n, k)
     assert ids.dtype == torch.long and int(ids.min()) >= 0 and int(ids.max()) < n
