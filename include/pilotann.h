@@ -244,17 +244,20 @@ int pa_traverse_refine(int64_t *out_I, float *out_D, int64_t *buf_I,
  * |x_j|^2 - 2 q_i . x_j, products in half precision with float accumulation,
  * unordered.  query_f16 and base_f16 hold m and n IEEE half rows of d
  * elements, d % 64 == 0 (pad rows with zeros), and must be readable up to the
- * next multiple of 128 rows (the kernel loads whole tiles; what the padding
- * rows hold does not matter); base_norm [n] are the squared lengths of the
- * base rows; n >= 1, and pa_knn_list_capacity() is 0 for any other `keep`.
- * Values must fit the half range: scale both sets by one factor first.  The base rows are
- * dealt to n_seg workgroups per 128 query rows (n_seg > 1 when m is too small
- * to fill the device); segment s of query i leaves its list at
+ * next multiple of pa_knn_tile_rows() (256) rows: the kernel loads whole tiles,
+ * and what the padding rows hold does not matter; base_norm [n] are the
+ * squared lengths of the base rows; n >= 1, and pa_knn_list_capacity() is 0
+ * for any other `keep`.  Values must fit the half range: scale both sets by
+ * one factor first.  The base rows are dealt to n_seg workgroups per tile of
+ * query rows (n_seg > 1 when m is too small to fill the device; a segment
+ * starts its lists from nothing, so many segments cost more than they
+ * spread); segment s of query i leaves its list at
  * cand_score / cand_id [(s * m + i) * pa_knn_list_capacity(keep)], of which
  * the first cand_count [s * m + i] (at most keep) entries are valid.  Device
  * pointers; enqueued on `stream`.
  */
 int64_t pa_knn_list_capacity(int keep);
+int pa_knn_tile_rows(void);
 int pa_knn(float *cand_score, int32_t *cand_id, int32_t *cand_count,
            const void *query_f16, const void *base_f16, const float *base_norm,
            int64_t m, int64_t n, int d, int keep, int n_seg, void *stream);

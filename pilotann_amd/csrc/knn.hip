@@ -7,21 +7,22 @@
 // fused with the selection, so the N x N table of scores never exists in
 // memory.  The caller ranks the candidates again with exact float distances.
 //
-// A workgroup of four wavefronts owns 128 query rows and walks over the base
-// rows 128 at a time.  Per 128 x 128 tile both operands go through LDS in
-// chunks of 64 elements (16-byte loads, the next chunk waiting in registers
-// while the present one is multiplied); a wavefront multiplies 64 x 64 of the
-// tile as 2 x 2 instructions tiles.  score(i, j) = |x_j|^2 - 2 q_i . x_j ranks
-// the base rows of query i like the squared distance does.
+// A workgroup of eight wavefronts owns 256 query rows and walks over the base
+// rows 256 at a time.  Per 256 x 256 tile both operands go through LDS in
+// chunks of 64 elements (16-byte loads; two staging buffers, the chunk after
+// the next waiting in registers); a wavefront multiplies 128 x 64 of the tile
+// as 4 x 2 instruction tiles.  score(i, j) = |x_j|^2 - 2 q_i . x_j ranks the
+// base rows of query i like the squared distance does.  With tiles of this
+// size every product moves 1/64 byte of operands through the memory system,
+// and that traffic, not the matrix cores, sets the pace.
 //
 // Selection: every query row has a list of (score, id) in device memory and,
-// in LDS, its length and a bound: the keep-th smallest score at the time the
-// list was last cut.  A score below the bound is appended (LDS atomic for the
-// position); once a list could overflow with the next tile, the wavefront
-// that owns the row cuts it to its `keep` smallest (a radix selection over
-// the order-preserving integer image of the scores, in registers) and lowers
-// the bound.  After the first few tiles almost nothing passes the bound, so
-// the matrix instructions are what the kernel spends its time on.
+// in LDS, its length and a limit from the keep-th smallest score at the time
+// the list was last cut.  A score below that bound is appended (LDS atomic
+// for the position); once a list could overflow with the next tile, the
+// wavefront that owns the row cuts it to its `keep` smallest (a radix
+// selection over the order-preserving integer image of the scores, in
+// registers) and moves the limit.  Late in the walk few scores pass.
 #include <hip/hip_runtime.h>
 #include <math.h>
 #include <stdint.h>
@@ -37,14 +38,14 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
 
-constexpr int kBM = 128;          // query rows per workgroup
-constexpr int kBN = 128;          // base rows per tile
 constexpr int kChunk = 64;        // contraction elements staged at a time
 // LDS row pitch in bytes: 128 of data + 16, so that consecutive rows start
 // four banks apart and the 16-byte reads of eight lanes cover every bank once
 constexpr int kPitch = kChunk * 2 + 16;
 constexpr int kSlack = 128;       // appended entries a list may hold beyond
                                   // `keep` before it must be cut
+constexpr int kMaxBN = 256;       // the most base rows a tile has in any form
+constexpr int kRowPad = 256;      // rows the caller's arrays are padded to
 
 struct KnnArgs {
     const _Float16 *query, *base;
@@ -63,12 +64,25 @@ __device__ __forceinline__ float unordered(unsigned u) {
     return __uint_as_float((u & 0x80000000u) ? (u & 0x7fffffffu) : ~u);
 }
 
-// The wavefront cuts one list of `n` entries (keep < n <= keep + kSlack + kBN)
+// The larger of two or three finite numbers (the plain instructions: fmaxf
+// first rewrites every operand that could be a signalling NaN).
+__device__ __forceinline__ float larger(float x, float y) {
+    float r;
+    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(x), "v"(y));
+    return r;
+}
+__device__ __forceinline__ float larger(float x, float y, float z) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "v"(y), "v"(z));
+    return r;
+}
+
+// The wavefront cuts one list of `n` entries (keep < n <= keep + kSlack + BN)
 // to its `keep` smallest, which end up in its first `keep` places, and returns
 // the largest score kept.
-template <int KEEP>
+template <int KEEP, int BN>
 __device__ __forceinline__ float cut_list(float *score, int32_t *id, int n, int lane) {
-    constexpr int kPerLane = (KEEP + kSlack + kBN + kWave - 1) / kWave;
+    constexpr int kPerLane = (KEEP + kSlack + BN + kWave - 1) / kWave;
     unsigned u[kPerLane];
     int32_t v[kPerLane];
 #pragma unroll
@@ -112,150 +126,219 @@ __device__ __forceinline__ float cut_list(float *score, int32_t *id, int n, int 
     return unordered(bound);
 }
 
-template <int KEEP>
-__global__ __launch_bounds__(256) void knn_kernel(KnnArgs a) {
-    constexpr int kCap = KEEP + kSlack + kBN;  // entries a list can hold
-    __shared__ __align__(16) unsigned char a_s[kBM * kPitch];
-    __shared__ __align__(16) unsigned char b_s[kBN * kPitch];
-    __shared__ int count[kBM];
-    __shared__ float bound[kBM];
+// WR x WC wavefronts, each multiplying WM x WN instruction tiles of 32 x 32:
+// the workgroup owns BM = 32 WR WM query rows and takes BN = 32 WC WN base
+// rows per tile.
+//
+// The sums start at -|x_j|^2 / 2 instead of zero, so a finished sum s is
+// -score / 2 and "score below the row's bound" is "s above the row's limit",
+// limit = -bound / 2: one comparison per product sum, and a row's sums over
+// the wavefront's columns are first reduced to their maximum.
+//
+// Chunks flow through two staging buffers without a break between tiles:
+// chunk c is multiplied out of buffer c % 2 while chunk c + 1 goes from the
+// registers into the other buffer and chunk c + 2 from memory into the
+// registers (one barrier per chunk); the chunk after a tile's last is the
+// first of the next tile.
+template <int KEEP, int WR, int WC, int WM, int WN>
+__global__ __launch_bounds__(64 * WR * WC, (WM * WN > 8 ? 1 : 2)) void knn_kernel(KnnArgs a) {
+    constexpr int kThreads = kWave * WR * WC;
+    constexpr int BM = 32 * WR * WM, BN = 32 * WC * WN;
+    constexpr int kStageRows = kThreads / 8;   // rows one staging step covers
+    constexpr int kOwnRows = BM / (WR * WC);   // lists a wavefront looks after
+    static_assert(BN <= kMaxBN && kRowPad % BM == 0 && kRowPad % BN == 0, "tile sizes");
+    static_assert(kOwnRows == 32 || kOwnRows == 64, "lists per wavefront");
+    static_assert(BM % kStageRows == 0 && BN % kStageRows == 0, "staging steps");
+    constexpr int kCap = KEEP + kSlack + kMaxBN;  // entries a list can hold
+    constexpr int kStepUnroll = WM * WN > 4 ? 1 : 2;
+    // a staging buffer: the chunk of the query tile, then that of the base tile
+    constexpr int kStage = (BM + BN) * kPitch;
+    __shared__ __align__(16) unsigned char stage[2 * kStage];
+    __shared__ int count[BM];
+    __shared__ float limit[BM];
     const int t = threadIdx.x;
     const int lane = t & (kWave - 1), wave = t / kWave;
+    const int wr = wave % WR, wc = wave / WR;
     const int col = lane & 31, half = lane >> 5;
-    const int64_t q0 = (int64_t)blockIdx.x * kBM;
+    const int64_t q0 = (int64_t)blockIdx.x * BM;
     const int seg = blockIdx.y;
     float *my_score = a.cand_score + ((size_t)seg * a.m + q0) * kCap;
     int32_t *my_id = a.cand_id + ((size_t)seg * a.m + q0) * kCap;
 
-    if (t < kBM) {
-        count[t] = 0;
-        bound[t] = q0 + t < a.m ? INFINITY : -INFINITY;  // rows past the end take nothing
+    for (int r = t; r < BM; r += kThreads) {
+        count[r] = 0;
+        limit[r] = q0 + r < a.m ? -INFINITY : INFINITY;  // rows past the end take nothing
     }
 
-    // staging: lane t copies 16-byte piece t % 8 of rows t / 8 + 32 i.  The
-    // caller's arrays are readable up to the next multiple of 128 rows, and a
-    // row is a whole number of chunks: no clamping, and addresses are a
-    // uniform base plus one 32-bit offset per lane
+    // staging: lane t copies 16-byte piece t % 8 of rows t / 8 + kStageRows i.
+    // The caller's arrays are readable up to the next multiple of kRowPad
+    // rows, and a row is a whole number of chunks: no clamping, and addresses
+    // are a uniform base plus one 32-bit offset per lane
     const int srow = t >> 3, spiece = t & 7;
     const unsigned lane_off = ((unsigned)srow * (unsigned)a.d + 8u * spiece) * 2u;
     const unsigned char *a_base =
         reinterpret_cast<const unsigned char *>(a.query) + (size_t)q0 * a.d * 2;
-    const unsigned char *a_tile = a_s + ((wave & 1) * 64 + col) * kPitch + 16 * half;
-    const unsigned char *b_tile = b_s + ((wave >> 1) * 64 + col) * kPitch + 16 * half;
-    const int64_t n_tiles = (a.n + kBN - 1) / kBN;
+    const unsigned char *a_tile = stage + (wr * WM * 32 + col) * kPitch + 16 * half;
+    const unsigned char *b_tile = stage + (BM + wc * WN * 32 + col) * kPitch + 16 * half;
+    unsigned char *my_stage = stage + srow * kPitch + 16 * spiece;
+    const int64_t n_tiles = (a.n + BN - 1) / BN;
+
+    uintx4 a_reg[BM / kStageRows], b_reg[BN / kStageRows];
+    int64_t f_tile = seg;   // the chunk the next fetch takes: tile and element
+    int f_k0 = 0;
+    bool pending;           // the registers hold a chunk that is not staged yet
+// the next chunk, if there is one, from memory into the registers
+#define PA_FETCH_NEXT                                                                   \
+    {                                                                                   \
+        pending = f_tile < n_tiles;                                                     \
+        if (pending) {                                                                  \
+            const unsigned char *b_from = reinterpret_cast<const unsigned char *>(      \
+                a.base) + ((size_t)f_tile * BN * a.d + f_k0) * 2;                       \
+            _Pragma("unroll") for (int i = 0; i < BM / kStageRows; ++i) a_reg[i] =      \
+                *reinterpret_cast<const uintx4 *>(                                      \
+                    a_base + ((size_t)(kStageRows * i) * a.d + f_k0) * 2 + lane_off);   \
+            _Pragma("unroll") for (int i = 0; i < BN / kStageRows; ++i) b_reg[i] =      \
+                *reinterpret_cast<const uintx4 *>(                                      \
+                    b_from + (size_t)(kStageRows * i) * a.d * 2 + lane_off);            \
+            f_k0 += kChunk;                                                             \
+            if (f_k0 >= a.d) f_k0 = 0, f_tile += a.n_seg;                               \
+        }                                                                               \
+    }
+// ... and from the registers into staging buffer `buf`
+#define PA_STORE_CHUNK(buf)                                                             \
+    {                                                                                   \
+        _Pragma("unroll") for (int i = 0; i < BM / kStageRows; ++i)                     \
+            *reinterpret_cast<uintx4 *>(                                                \
+                my_stage + (buf) * kStage + kStageRows * i * kPitch) = a_reg[i];        \
+        _Pragma("unroll") for (int i = 0; i < BN / kStageRows; ++i)                     \
+            *reinterpret_cast<uintx4 *>(                                                \
+                my_stage + (buf) * kStage + (BM + kStageRows * i) * kPitch) = b_reg[i]; \
+    }
+// minus half the squared lengths of a tile's base rows, the columns of this
+// wavefront (a column past the end: minus infinity, so it never passes)
+#define PA_LOAD_NORMS(tile_)                                                            \
+    _Pragma("unroll") for (int n = 0; n < WN; ++n) {                                    \
+        const int64_t c = (tile_) * BN + (wc * WN + n) * 32 + col;                      \
+        start[n] = c < a.n ? -0.5f * a.base_norm[c] : -INFINITY;                        \
+    }
+    float start[WN];
+    if (seg < n_tiles) PA_LOAD_NORMS((int64_t)seg)
+    PA_FETCH_NEXT
+    PA_STORE_CHUNK(0)
+    PA_FETCH_NEXT
     __syncthreads();
+    int buf = 0;
 
     for (int64_t tile = seg; tile < n_tiles; tile += a.n_seg) {
-        const int64_t n0 = tile * kBN;
-        const unsigned char *b_base =
-            reinterpret_cast<const unsigned char *>(a.base) + (size_t)n0 * a.d * 2;
-        floatx16 acc[2][2];
+        floatx16 acc[WM][WN];
 #pragma unroll
-        for (int m = 0; m < 2; ++m)
+        for (int m = 0; m < WM; ++m)
 #pragma unroll
-            for (int n = 0; n < 2; ++n)
+            for (int n = 0; n < WN; ++n)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) acc[m][n][r] = 0.f;
+                for (int r = 0; r < 16; ++r) acc[m][n][r] = start[n];
 
-        uintx4 a_reg[kBM / 32], b_reg[kBN / 32];
-// the chunk that starts at element k0, from memory into registers
-#define PA_FETCH_CHUNK(k0)                                                              \
-    {                                                                                   \
-        _Pragma("unroll") for (int i = 0; i < kBM / 32; ++i) a_reg[i] =                 \
-            *reinterpret_cast<const uintx4 *>(                                          \
-                a_base + ((size_t)(32 * i) * a.d + (k0)) * 2 + lane_off);               \
-        _Pragma("unroll") for (int i = 0; i < kBN / 32; ++i) b_reg[i] =                 \
-            *reinterpret_cast<const uintx4 *>(                                          \
-                b_base + ((size_t)(32 * i) * a.d + (k0)) * 2 + lane_off);               \
-    }
-        PA_FETCH_CHUNK(0)
 #pragma unroll 1
-        for (int k0 = 0; k0 < a.d; k0 += kChunk) {
-#pragma unroll
-            for (int i = 0; i < kBM / 32; ++i)
-                *reinterpret_cast<uintx4 *>(a_s + (srow + 32 * i) * kPitch + 16 * spiece) = a_reg[i];
-#pragma unroll
-            for (int i = 0; i < kBN / 32; ++i)
-                *reinterpret_cast<uintx4 *>(b_s + (srow + 32 * i) * kPitch + 16 * spiece) = b_reg[i];
-            __syncthreads();
-            if (k0 + kChunk < a.d) PA_FETCH_CHUNK(k0 + kChunk)
+        for (int k0 = 0; k0 < a.d; k0 += kChunk, buf ^= 1) {
+            if (pending) {
+                PA_STORE_CHUNK(buf ^ 1)
+                PA_FETCH_NEXT
+            }
             // MFMA operands: lane l supplies eight consecutive elements of row
             // l % 32, the first or second eight of a group of 16 by l / 32 —
             // the same for both operands, which is all the sum needs
-#pragma unroll 2
+            const unsigned char *a_now = a_tile + buf * kStage, *b_now = b_tile + buf * kStage;
+#pragma unroll kStepUnroll
             for (int s = 0; s < kChunk / 16; ++s) {
-                half8 av[2], bv[2];
+                half8 av[WM], bv[WN];
 #pragma unroll
-                for (int m = 0; m < 2; ++m)
-                    av[m] = *reinterpret_cast<const half8 *>(a_tile + m * 32 * kPitch + 32 * s);
+                for (int m = 0; m < WM; ++m)
+                    av[m] = *reinterpret_cast<const half8 *>(a_now + m * 32 * kPitch + 32 * s);
 #pragma unroll
-                for (int n = 0; n < 2; ++n)
-                    bv[n] = *reinterpret_cast<const half8 *>(b_tile + n * 32 * kPitch + 32 * s);
+                for (int n = 0; n < WN; ++n)
+                    bv[n] = *reinterpret_cast<const half8 *>(b_now + n * 32 * kPitch + 32 * s);
 #pragma unroll
-                for (int m = 0; m < 2; ++m)
+                for (int m = 0; m < WM; ++m)
 #pragma unroll
-                    for (int n = 0; n < 2; ++n)
+                    for (int n = 0; n < WN; ++n)
                         acc[m][n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
                             av[m], bv[n], acc[m][n], 0, 0, 0);
             }
             __syncthreads();
         }
-#undef PA_FETCH_CHUNK
 
+        // the next tile's norms travel while this tile's sums are looked at
+        if (tile + a.n_seg < n_tiles) PA_LOAD_NORMS(tile + a.n_seg)
         // a lane's 16 results of an instruction tile are
         // D[i = 8 * (r / 4) + 4 * (l / 32) + r % 4][j = l % 32]
+        const int32_t c0 = (int32_t)(tile * BN) + wc * WN * 32 + col;
 #pragma unroll
-        for (int n = 0; n < 2; ++n) {
-            const int64_t cg = n0 + (wave >> 1) * 64 + n * 32 + col;
-            const bool col_ok = cg < a.n;
-            const float xn = col_ok ? a.base_norm[cg] : 0.f;
+        for (int m = 0; m < WM; ++m) {
+            // one row of instruction tiles at a time, so that its limits and
+            // sums are all that is live
+            __builtin_amdgcn_sched_barrier(0);
+            const int row0 = (wr * WM + m) * 32 + 4 * half;
+            float lim[16];
 #pragma unroll
-            for (int m = 0; m < 2; ++m) {
+            for (int r = 0; r < 16; ++r) lim[r] = limit[row0 + 8 * (r >> 2) + (r & 3)];
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int row = (wave & 1) * 64 + m * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
-                    const float sc = fmaf(-2.f, acc[m][n][r], xn);
-                    const bool pass = col_ok && sc < bound[row];
-                    if (__ballot(pass)) {  // rare after the first tiles
-                        if (pass) {
-                            const int pos = atomicAdd(&count[row], 1);
-                            my_score[(size_t)row * kCap + pos] = sc;
-                            my_id[(size_t)row * kCap + pos] = (int32_t)cg;
+            for (int r = 0; r < 16; ++r) {
+                float best = acc[m][0][r];
+                if constexpr (WN == 4) {
+                    best = larger(larger(best, acc[m][1][r], acc[m][2][r]), acc[m][3][r]);
+                } else {
+#pragma unroll
+                    for (int n = 1; n < WN; ++n) best = larger(best, acc[m][n][r]);
+                }
+                if (best > lim[r]) {  // rare after the first tiles
+                    const int row = row0 + 8 * (r >> 2) + (r & 3);
+#pragma unroll
+                    for (int n = 0; n < WN; ++n) {
+                        if (acc[m][n][r] > lim[r]) {
+                            const unsigned at = row * kCap + atomicAdd(&count[row], 1);
+                            my_score[at] = -2.f * acc[m][n][r];
+                            my_id[at] = c0 + 32 * n;
                         }
                     }
                 }
             }
         }
         __syncthreads();
-        // wavefront w looks after rows 32 w .. 32 w + 31: a list that the
-        // next tile could overflow is cut now
+        // every wavefront looks after kOwnRows lists: one that the next tile
+        // could overflow is cut now
         {
-            const int row = wave * 32 + col;
-            unsigned long long todo = __ballot(half == 0 && count[row] > KEEP + kSlack);
+            const int row = wave * kOwnRows + lane % kOwnRows;
+            unsigned long long todo =
+                __ballot(lane < kOwnRows && count[row] > KEEP + kSlack);
             while (todo) {
-                const int r = wave * 32 + __builtin_ctzll(todo);
+                const int r = wave * kOwnRows + __builtin_ctzll(todo);
                 todo &= todo - 1;
-                const float b = cut_list<KEEP>(my_score + (size_t)r * kCap,
-                                               my_id + (size_t)r * kCap, count[r], lane);
-                if (lane == 0) count[r] = KEEP, bound[r] = b;
+                const float b = cut_list<KEEP, BN>(my_score + (size_t)r * kCap,
+                                                   my_id + (size_t)r * kCap, count[r], lane);
+                if (lane == 0) count[r] = KEEP, limit[r] = -0.5f * b;
             }
         }
         // the next tile's first barrier comes before anything reads the
-        // counts and bounds again
+        // counts and limits again
     }
+#undef PA_FETCH_NEXT
+#undef PA_STORE_CHUNK
+#undef PA_LOAD_NORMS
     __syncthreads();
     {
-        const int row = wave * 32 + col;
-        unsigned long long todo = __ballot(half == 0 && count[row] > KEEP);
+        const int row = wave * kOwnRows + lane % kOwnRows;
+        unsigned long long todo = __ballot(lane < kOwnRows && count[row] > KEEP);
         while (todo) {
-            const int r = wave * 32 + __builtin_ctzll(todo);
+            const int r = wave * kOwnRows + __builtin_ctzll(todo);
             todo &= todo - 1;
-            cut_list<KEEP>(my_score + (size_t)r * kCap, my_id + (size_t)r * kCap, count[r], lane);
+            cut_list<KEEP, BN>(my_score + (size_t)r * kCap, my_id + (size_t)r * kCap,
+                               count[r], lane);
             if (lane == 0) count[r] = KEEP;
         }
     }
     __syncthreads();
-    if (t < kBM && q0 + t < a.m) a.cand_count[(size_t)seg * a.m + q0 + t] = count[t];
+    for (int r = t; r < BM; r += kThreads)
+        if (q0 + r < a.m) a.cand_count[(size_t)seg * a.m + q0 + r] = count[r];
 }
 
 // Occlusion pruning of a node's candidate list (closest first): candidate j
@@ -310,11 +393,26 @@ __global__ __launch_bounds__(256) void prune_kernel(
     for (int i = count + lane; i < m_keep; i += kWave) out[i] = -1;
 }
 
+// The form in use: 2 x 4 wavefronts of 4 x 2 instruction tiles, 256 query rows
+// against 256 base rows per tile; one workgroup per compute unit (150 KB of
+// LDS, 256 registers a lane).
+constexpr int kWR = 2, kWC = 4, kWM = 4, kWN = 2;
+constexpr int kBM = 32 * kWR * kWM;
+
+template <int KEEP>
+int launch_knn(const KnnArgs &a, hipStream_t stream) {
+    const dim3 grid((unsigned)((a.m + kBM - 1) / kBM), (unsigned)a.n_seg);
+    knn_kernel<KEEP, kWR, kWC, kWM, kWN><<<grid, 64 * kWR * kWC, 0, stream>>>(a);
+    return (int)hipGetLastError();
+}
+
 }  // namespace
 
 extern "C" int64_t pa_knn_list_capacity(int keep) {
-    return keep == 64 || keep == 128 || keep == 256 || keep == 512 ? keep + kSlack + kBN : 0;
+    return keep == 64 || keep == 128 || keep == 256 || keep == 512 ? keep + kSlack + kMaxBN : 0;
 }
+
+extern "C" int pa_knn_tile_rows(void) { return kRowPad; }
 
 extern "C" int pa_knn(float *cand_score, int32_t *cand_id, int32_t *cand_count,
                       const void *query_f16, const void *base_f16,
@@ -334,15 +432,13 @@ extern "C" int pa_knn(float *cand_score, int32_t *cand_id, int32_t *cand_count,
     a.base_norm = base_norm;
     a.cand_score = cand_score, a.cand_id = cand_id, a.cand_count = cand_count;
     a.m = m, a.n = n, a.d = d, a.n_seg = n_seg;
-    const dim3 grid((unsigned)((m + kBM - 1) / kBM), (unsigned)n_seg);
     hipStream_t stream = (hipStream_t)stream_;
     switch (keep) {
-        case 64: knn_kernel<64><<<grid, 256, 0, stream>>>(a); break;
-        case 128: knn_kernel<128><<<grid, 256, 0, stream>>>(a); break;
-        case 256: knn_kernel<256><<<grid, 256, 0, stream>>>(a); break;
-        default: knn_kernel<512><<<grid, 256, 0, stream>>>(a);
+        case 64: return launch_knn<64>(a, stream);
+        case 128: return launch_knn<128>(a, stream);
+        case 256: return launch_knn<256>(a, stream);
+        default: return launch_knn<512>(a, stream);
     }
-    return (int)hipGetLastError();
 }
 
 extern "C" int pa_graph_prune(int32_t *selected, const float *pair,

@@ -302,9 +302,9 @@ def entry_distances(query: torch.Tensor, entry_vectors: torch.Tensor):
 
 class HalfRows:
     """Rows prepared for :func:`knn_candidates`: a half-precision copy, scaled
-    into [-1, 1], padded with zeros to a multiple of 128 rows and 64 columns
-    (what the kernel reads without bounds checks), and the squared lengths of
-    the scaled rows."""
+    into [-1, 1], padded with zeros to whole tiles of the kernel
+    (``pa_knn_tile_rows()`` rows, 64 columns: what it reads without bounds
+    checks), and the squared lengths of the scaled rows."""
 
     def __init__(self, rows: torch.Tensor, scale: float = None):
         _check(rows, 'rows', 2, torch.float32, True)
@@ -312,7 +312,8 @@ class HalfRows:
         if scale is None:
             scale = 1.0 / max(float(rows.abs().max()), 1e-30) if n else 1.0
         self.n, self.d, self.scale = n, d, scale
-        n_pad, d_pad = -(-max(n, 1) // 128) * 128, -(-d // 64) * 64
+        self.tile = int(_lib.lib().pa_knn_tile_rows())
+        n_pad, d_pad = -(-max(n, 1) // self.tile) * self.tile, -(-d // 64) * 64
         self.half = torch.zeros(n_pad, d_pad, dtype=torch.float16, device=rows.device)
         self.half[:n, :d] = rows * scale
         self.norm = torch.zeros(n_pad, dtype=torch.float32, device=rows.device)
@@ -320,12 +321,17 @@ class HalfRows:
 
     def rows(self, lo: int, hi: int) -> 'HalfRows':
         """Rows ``lo .. hi`` as a set of their own (a view; ``lo`` a multiple
-        of 128, so that the padding still reaches a whole tile)."""
-        _require(lo % 128 == 0 and 0 <= lo < hi <= self.n, 'lo % 128 == 0, lo < hi <= n')
+        of the tile, so that the padding still reaches a whole tile)."""
+        _require(lo % self.tile == 0 and 0 <= lo < hi <= self.n,
+                 'lo a multiple of the tile rows, lo < hi <= n')
         part = HalfRows.__new__(HalfRows)
-        part.n, part.d, part.scale = hi - lo, self.d, self.scale
+        part.n, part.d, part.scale, part.tile = hi - lo, self.d, self.scale, self.tile
         part.half, part.norm = self.half[lo:], self.norm[lo:]
         return part
+
+
+# workgroups the device runs at a time: one per compute unit
+_KNN_RESIDENT = 256
 
 
 def knn_candidates(query, base, keep: int, n_seg: int = None):
@@ -346,10 +352,11 @@ def knn_candidates(query, base, keep: int, n_seg: int = None):
     m, n, device = query.n, base.n, base.half.device
     if m == 0:
         return torch.empty(0, keep, dtype=torch.long, device=device)
+    tile = query.tile
+    blocks, tiles = -(-m // tile), -(-n // tile)
     if n_seg is None:
-        # enough workgroups for two per compute unit
-        blocks, tiles = -(-m // 128), -(-n // 128)
-        n_seg = max(1, min(tiles, -(-512 // blocks)))
+        # enough workgroups for one per compute unit
+        n_seg = max(1, min(tiles, _KNN_RESIDENT // blocks))
     cap = int(_lib.lib().pa_knn_list_capacity(int(keep)))
     _require(cap > 0, 'keep is 64, 128, 256 or 512')
     score = torch.empty(n_seg, m, cap, dtype=torch.float32, device=device)

@@ -69,8 +69,8 @@ def test_the_device_table_agrees_with_the_host_path(device):
     (200, 9000, 64, 256), (130, 5000, 96, 512),
 ])
 def test_candidates_of_a_few_queries_over_segments(m, n, d, keep, device):
-    """Few query rows: the base rows are dealt to several workgroups per 128
-    queries and the lists merged; the exact nearest keep / 2 rows must be
+    """Few query rows: the base rows are dealt to several workgroups per tile
+    of queries and the lists merged; the exact nearest keep / 2 rows must be
     among the keep candidates."""
     print('knn candidates', m, n, d, keep, flush=True)
     g = torch.Generator().manual_seed(m + n)
@@ -85,8 +85,24 @@ def test_candidates_of_a_few_queries_over_segments(m, n, d, keep, device):
     assert overlap(cand, want) > 0.9995
     # one segment and many give the same sets when nothing is tied
     one = kernels.knn_candidates(query, base, keep, n_seg=1)
-    many = kernels.knn_candidates(query, base, keep, n_seg=min(7, -(-n // 128)))
+    many = kernels.knn_candidates(query, base, keep, n_seg=min(7, -(-n // 256)))
     assert overlap(one, want) > 0.9995 and overlap(many, want) > 0.9995
+
+
+def test_a_part_of_a_prepared_set_as_queries(device):
+    """Query rows taken from a prepared set (a view that starts on a tile)
+    against the whole set."""
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(3000, 64, generator=g).to(device)
+    rows = kernels.HalfRows(x)
+    print('knn candidates, rows 512 .. 3000 of a prepared set', flush=True)
+    part = kernels.knn_candidates(rows.rows(512, 3000), rows, 64)
+    torch.cuda.synchronize()
+    assert part.shape == (2488, 64)
+    want = exact_neighbours(x[512:], x, 32).indices
+    assert overlap(part, want) > 0.9995
+    with pytest.raises(RuntimeError):
+        rows.rows(100, 3000)
 
 
 def test_fewer_base_rows_than_candidates(device):
@@ -129,8 +145,9 @@ def test_knn_argument_errors(device):
     assert call(m=-1) != 0
     assert call(q=none) != 0
     assert call(m=0) == 0
-    assert lib.pa_knn_list_capacity(64) == 320 and lib.pa_knn_list_capacity(128) == 384
-    assert lib.pa_knn_list_capacity(512) == 768 and lib.pa_knn_list_capacity(100) == 0
+    assert lib.pa_knn_tile_rows() == 256
+    assert lib.pa_knn_list_capacity(64) == 448 and lib.pa_knn_list_capacity(128) == 512
+    assert lib.pa_knn_list_capacity(512) == 896 and lib.pa_knn_list_capacity(100) == 0
     with pytest.raises(RuntimeError):
         kernels.knn_candidates(torch.zeros(4, 64), torch.zeros(200, 64, device=device), 64)
     with pytest.raises(RuntimeError):
