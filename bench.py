@@ -64,7 +64,7 @@ CONFIGS = {
     # minutes: the subgraph on a seeded random quarter of the nodes and no
     # full graph, hence no refine and no end-to-end recall (the recall
     # reported is that of the candidate lists); --full-index builds the whole
-    # index (six minutes) and measures the whole search.
+    # index (four minutes) and measures the whole search.
     'c5': dict(n=10_000_000, d=768, dp=128, n_centers=4096, sigma=1.0,
                decay=0.0, normalize=True, ratio=0.25, graph='nsg48',
                entry='router64x64', queries=10_000, k=10, ef_sweep=[128],
