@@ -9,12 +9,12 @@
 //
 // A workgroup of eight wavefronts owns 256 query rows and walks over the base
 // rows 256 at a time.  Per 256 x 256 tile both operands go through LDS in
-// chunks of 64 elements (16-byte loads; two staging buffers, the chunk after
-// the next waiting in registers); a wavefront multiplies 128 x 64 of the tile
-// as 4 x 2 instruction tiles.  score(i, j) = |x_j|^2 - 2 q_i . x_j ranks the
-// base rows of query i like the squared distance does.  With tiles of this
-// size every product moves 1/64 byte of operands through the memory system,
-// and that traffic, not the matrix cores, sets the pace.
+// chunks of 64 elements, loaded from memory straight into two staging
+// buffers; a wavefront multiplies 128 x 64 of the tile as 4 x 2 instruction
+// tiles.  score(i, j) = |x_j|^2 - 2 q_i . x_j ranks the base rows of query i
+// like the squared distance does.  With tiles of this size every product
+// moves 1/64 byte of operands through the memory system, and that traffic,
+// not the matrix cores, sets the pace.
 //
 // Selection: every query row has a list of (score, id) in device memory and,
 // in LDS, its length and a limit from the keep-th smallest score at the time
@@ -38,10 +38,8 @@ typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
 
-constexpr int kChunk = 64;        // contraction elements staged at a time
-// LDS row pitch in bytes: 128 of data + 16, so that consecutive rows start
-// four banks apart and the 16-byte reads of eight lanes cover every bank once
-constexpr int kPitch = kChunk * 2 + 16;
+constexpr int kChunk = 64;        // contraction elements staged at a time; a
+                                  // row is a whole number of chunks
 constexpr int kSlack = 128;       // appended entries a list may hold beyond
                                   // `keep` before it must be cut
 constexpr int kMaxBN = 256;       // the most base rows a tile has in any form
@@ -75,6 +73,19 @@ __device__ __forceinline__ float larger(float x, float y, float z) {
     float r;
     asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(x), "v"(y), "v"(z));
     return r;
+}
+
+// Every lane's 16 bytes at `from` go to LDS, side by side from `lds_addr` (the
+// same for all lanes) on.  The compiler does not know of the transfer: the
+// wavefront waits with bring_wait() before a barrier makes the rows public.
+__device__ __forceinline__ void bring_rows(const void *from, unsigned lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off"
+                 :: "s"(__builtin_amdgcn_readfirstlane(lds_addr)), "v"(from)
+                 : "memory", "m0");
+}
+template <int LEFT>   // until at most LEFT of the wavefront's transfers are under way
+__device__ __forceinline__ void bring_wait() {
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(LEFT) : "memory");
 }
 
 // The wavefront cuts one list of `n` entries (keep < n <= keep + kSlack + BN)
@@ -135,11 +146,11 @@ __device__ __forceinline__ float cut_list(float *score, int32_t *id, int n, int 
 // limit = -bound / 2: one comparison per product sum, and a row's sums over
 // the wavefront's columns are first reduced to their maximum.
 //
-// Chunks flow through two staging buffers without a break between tiles:
-// chunk c is multiplied out of buffer c % 2 while chunk c + 1 goes from the
-// registers into the other buffer and chunk c + 2 from memory into the
-// registers (one barrier per chunk); the chunk after a tile's last is the
-// first of the next tile.
+// Chunks flow through a ring of staging buffers without a break between
+// tiles: chunk c is multiplied out of buffer c % 2 while chunk c + 1 travels
+// from memory straight into the other buffer (global_load_lds, 16 bytes a
+// lane; no registers and no LDS stores in between); one barrier per chunk; the
+// chunk after a tile's last is the first of the next tile.
 template <int KEEP, int WR, int WC, int WM, int WN>
 __global__ __launch_bounds__(64 * WR * WC, (WM * WN > 8 ? 1 : 2)) void knn_kernel(KnnArgs a) {
     constexpr int kThreads = kWave * WR * WC;
@@ -150,10 +161,25 @@ __global__ __launch_bounds__(64 * WR * WC, (WM * WN > 8 ? 1 : 2)) void knn_kerne
     static_assert(kOwnRows == 32 || kOwnRows == 64, "lists per wavefront");
     static_assert(BM % kStageRows == 0 && BN % kStageRows == 0, "staging steps");
     constexpr int kCap = KEEP + kSlack + kMaxBN;  // entries a list can hold
-    constexpr int kStepUnroll = WM * WN > 4 ? 1 : 2;
-    // a staging buffer: the chunk of the query tile, then that of the base tile
-    constexpr int kStage = (BM + BN) * kPitch;
-    __shared__ __align__(16) unsigned char stage[2 * kStage];
+    // a staging buffer: the chunk of the query tile, then that of the base
+    // tile, rows of kRow bytes without padding; the 16-byte piece p of row r
+    // lies at place p ^ (r % 8) of its row, so that neither the loads that
+    // fill the buffer nor the operand reads meet in a bank
+    constexpr int kRow = kChunk * 2;
+    constexpr int kPieces = kRow / 16;             // 16-byte pieces of a row
+    constexpr int kInstrRows = kWave / kPieces;    // rows one instruction brings
+    constexpr int kStage = (BM + BN) * kRow;
+    constexpr int kStages = (128 << 10) / kStage;  // buffers in the ring
+    constexpr int kWaves = WR * WC;
+    constexpr int kWaveRows = (BM + BN) / kWaves;  // rows a wavefront brings in per chunk
+    constexpr int kInstrs = kWaveRows / kInstrRows;
+    static_assert(kPieces == 8 || kPieces == 4, "chunk size");
+    static_assert(kStages >= 2 && kWaveRows % kInstrRows == 0 && BM % kWaveRows == 0,
+                  "rows per wavefront");
+    // transfers that may still be under way when the chunk needed next must
+    // be there: those of the chunks after it
+    constexpr int kAhead = kInstrs * (kStages - 2);
+    __shared__ __align__(1024) unsigned char stage[kStages * kStage];
     __shared__ int count[BM];
     __shared__ float limit[BM];
     const int t = threadIdx.x;
@@ -170,49 +196,47 @@ __global__ __launch_bounds__(64 * WR * WC, (WM * WN > 8 ? 1 : 2)) void knn_kerne
         limit[r] = q0 + r < a.m ? -INFINITY : INFINITY;  // rows past the end take nothing
     }
 
-    // staging: lane t copies 16-byte piece t % 8 of rows t / 8 + kStageRows i.
+    // staging goes from memory straight into LDS: one instruction of a
+    // wavefront brings 8 rows of a chunk, lane l the piece (l % 8) ^ (l / 8) of
+    // row l / 8, and the hardware puts the lanes' 16 bytes side by side.
     // The caller's arrays are readable up to the next multiple of kRowPad
-    // rows, and a row is a whole number of chunks: no clamping, and addresses
-    // are a uniform base plus one 32-bit offset per lane
-    const int srow = t >> 3, spiece = t & 7;
-    const unsigned lane_off = ((unsigned)srow * (unsigned)a.d + 8u * spiece) * 2u;
+    // rows, and a row is a whole number of chunks: no clamping
+    const int my_first = wave * kWaveRows;      // among the BM + BN rows of a buffer
+    const bool brings_query = my_first < BM;
+    const int bring_row = lane / kPieces;
+    const unsigned bring_off =
+        ((unsigned)((brings_query ? my_first : my_first - BM) + bring_row) * (unsigned)a.d) * 2u +
+        16u * ((lane % kPieces) ^ ((bring_row / (8 / kPieces)) & (kPieces - 1)));
     const unsigned char *a_base =
         reinterpret_cast<const unsigned char *>(a.query) + (size_t)q0 * a.d * 2;
-    const unsigned char *a_tile = stage + (wr * WM * 32 + col) * kPitch + 16 * half;
-    const unsigned char *b_tile = stage + (BM + wc * WN * 32 + col) * kPitch + 16 * half;
-    unsigned char *my_stage = stage + srow * kPitch + 16 * spiece;
+    const unsigned bring_to =
+        (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)stage + my_first * kRow;
+    // operand reads: lane l wants elements 16 s + 8 (l / 32) .. + 8 of row
+    // l % 32 of an instruction tile, piece 2 s + l / 32 of that row
+    const unsigned mix = (col / (8 / kPieces)) & (kPieces - 1);
+    const unsigned swizzle = 16u * (half ^ (mix & 1)) + 32u * (mix >> 1);
+    const unsigned char *a_tile = stage + (wr * WM * 32 + col) * kRow;
+    const unsigned char *b_tile = stage + (BM + wc * WN * 32 + col) * kRow;
     const int64_t n_tiles = (a.n + BN - 1) / BN;
 
-    uintx4 a_reg[BM / kStageRows], b_reg[BN / kStageRows];
     int64_t f_tile = seg;   // the chunk the next fetch takes: tile and element
     int f_k0 = 0;
-    bool pending;           // the registers hold a chunk that is not staged yet
-// the next chunk, if there is one, from memory into the registers
-#define PA_FETCH_NEXT                                                                   \
+    bool pending;           // a chunk is on its way into the other buffer
+// the next chunk, if there is one, from memory into staging buffer `buf`
+#define PA_FETCH_NEXT(buf)                                                              \
     {                                                                                   \
         pending = f_tile < n_tiles;                                                     \
         if (pending) {                                                                  \
-            const unsigned char *b_from = reinterpret_cast<const unsigned char *>(      \
-                a.base) + ((size_t)f_tile * BN * a.d + f_k0) * 2;                       \
-            _Pragma("unroll") for (int i = 0; i < BM / kStageRows; ++i) a_reg[i] =      \
-                *reinterpret_cast<const uintx4 *>(                                      \
-                    a_base + ((size_t)(kStageRows * i) * a.d + f_k0) * 2 + lane_off);   \
-            _Pragma("unroll") for (int i = 0; i < BN / kStageRows; ++i) b_reg[i] =      \
-                *reinterpret_cast<const uintx4 *>(                                      \
-                    b_from + (size_t)(kStageRows * i) * a.d * 2 + lane_off);            \
+            const unsigned char *from =                                                 \
+                (brings_query ? a_base + (size_t)f_k0 * 2                               \
+                              : reinterpret_cast<const unsigned char *>(a.base) +       \
+                                    ((size_t)f_tile * BN * a.d + f_k0) * 2) + bring_off;\
+            _Pragma("unroll") for (int i = 0; i < kInstrs; ++i)                         \
+                bring_rows(from + (size_t)(kInstrRows * i) * a.d * 2,                   \
+                           bring_to + (buf) * kStage + kInstrRows * i * kRow);          \
             f_k0 += kChunk;                                                             \
             if (f_k0 >= a.d) f_k0 = 0, f_tile += a.n_seg;                               \
         }                                                                               \
-    }
-// ... and from the registers into staging buffer `buf`
-#define PA_STORE_CHUNK(buf)                                                             \
-    {                                                                                   \
-        _Pragma("unroll") for (int i = 0; i < BM / kStageRows; ++i)                     \
-            *reinterpret_cast<uintx4 *>(                                                \
-                my_stage + (buf) * kStage + kStageRows * i * kPitch) = a_reg[i];        \
-        _Pragma("unroll") for (int i = 0; i < BN / kStageRows; ++i)                     \
-            *reinterpret_cast<uintx4 *>(                                                \
-                my_stage + (buf) * kStage + (BM + kStageRows * i) * kPitch) = b_reg[i]; \
     }
 // minus half the squared lengths of a tile's base rows, the columns of this
 // wavefront (a column past the end: minus infinity, so it never passes)
@@ -223,9 +247,9 @@ __global__ __launch_bounds__(64 * WR * WC, (WM * WN > 8 ? 1 : 2)) void knn_kerne
     }
     float start[WN];
     if (seg < n_tiles) PA_LOAD_NORMS((int64_t)seg)
-    PA_FETCH_NEXT
-    PA_STORE_CHUNK(0)
-    PA_FETCH_NEXT
+#pragma unroll
+    for (int b = 0; b < kStages - 1; ++b) PA_FETCH_NEXT(b)
+    if (pending) bring_wait<kAhead>(); else bring_wait<0>();
     __syncthreads();
     int buf = 0;
 
@@ -239,24 +263,23 @@ __global__ __launch_bounds__(64 * WR * WC, (WM * WN > 8 ? 1 : 2)) void knn_kerne
                 for (int r = 0; r < 16; ++r) acc[m][n][r] = start[n];
 
 #pragma unroll 1
-        for (int k0 = 0; k0 < a.d; k0 += kChunk, buf ^= 1) {
-            if (pending) {
-                PA_STORE_CHUNK(buf ^ 1)
-                PA_FETCH_NEXT
-            }
+        for (int k0 = 0; k0 < a.d; k0 += kChunk, buf = (buf + 1) % kStages) {
+            // nobody reads the other buffer any more: the next chunk goes there
+            PA_FETCH_NEXT((buf + kStages - 1) % kStages)
             // MFMA operands: lane l supplies eight consecutive elements of row
             // l % 32, the first or second eight of a group of 16 by l / 32 —
             // the same for both operands, which is all the sum needs
             const unsigned char *a_now = a_tile + buf * kStage, *b_now = b_tile + buf * kStage;
-#pragma unroll kStepUnroll
+#pragma unroll
             for (int s = 0; s < kChunk / 16; ++s) {
                 half8 av[WM], bv[WN];
+                const unsigned at = swizzle ^ (32u * s);
 #pragma unroll
                 for (int m = 0; m < WM; ++m)
-                    av[m] = *reinterpret_cast<const half8 *>(a_now + m * 32 * kPitch + 32 * s);
+                    av[m] = *reinterpret_cast<const half8 *>(a_now + m * 32 * kRow + at);
 #pragma unroll
                 for (int n = 0; n < WN; ++n)
-                    bv[n] = *reinterpret_cast<const half8 *>(b_now + n * 32 * kPitch + 32 * s);
+                    bv[n] = *reinterpret_cast<const half8 *>(b_now + n * 32 * kRow + at);
 #pragma unroll
                 for (int m = 0; m < WM; ++m)
 #pragma unroll
@@ -264,6 +287,7 @@ __global__ __launch_bounds__(64 * WR * WC, (WM * WN > 8 ? 1 : 2)) void knn_kerne
                         acc[m][n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
                             av[m], bv[n], acc[m][n], 0, 0, 0);
             }
+            if (pending) bring_wait<kAhead>(); else bring_wait<0>();
             __syncthreads();
         }
 
@@ -322,7 +346,6 @@ __global__ __launch_bounds__(64 * WR * WC, (WM * WN > 8 ? 1 : 2)) void knn_kerne
         // counts and limits again
     }
 #undef PA_FETCH_NEXT
-#undef PA_STORE_CHUNK
 #undef PA_LOAD_NORMS
     __syncthreads();
     {
