@@ -162,10 +162,13 @@ __global__ __launch_bounds__(64 * WR * WC, (WM * WN > 8 ? 1 : 2)) void knn_kerne
     static_assert(BM % kStageRows == 0 && BN % kStageRows == 0, "staging steps");
     constexpr int kCap = KEEP + kSlack + kMaxBN;  // entries a list can hold
     // a staging buffer: the chunk of the query tile, then that of the base
-    // tile, rows of kRow bytes without padding; the 16-byte piece p of row r
-    // lies at place p ^ (r % 8) of its row, so that neither the loads that
-    // fill the buffer nor the operand reads meet in a bank
+    // tile, rows of kRow bytes without padding.  LDS has 64 banks of four
+    // bytes and serves a 16-byte read to 16 lanes at a time: 16 consecutive
+    // rows are 8 pairs that share a 256-byte span, so the 16-byte piece p of
+    // row r lies at place p ^ ((r / 2) % 8) of its row, and neither the loads
+    // that fill the buffer nor the operand reads meet in a bank
     constexpr int kRow = kChunk * 2;
+#define PA_PLACE_MIX(row_) ((unsigned)((row_) / (256 / kRow)) & (unsigned)(kPieces - 1))
     constexpr int kPieces = kRow / 16;             // 16-byte pieces of a row
     constexpr int kInstrRows = kWave / kPieces;    // rows one instruction brings
     constexpr int kStage = (BM + BN) * kRow;
@@ -197,23 +200,23 @@ __global__ __launch_bounds__(64 * WR * WC, (WM * WN > 8 ? 1 : 2)) void knn_kerne
     }
 
     // staging goes from memory straight into LDS: one instruction of a
-    // wavefront brings 8 rows of a chunk, lane l the piece (l % 8) ^ (l / 8) of
-    // row l / 8, and the hardware puts the lanes' 16 bytes side by side.
+    // wavefront brings kInstrRows rows of a chunk, lane l a piece of row
+    // l / kPieces, the piece that belongs at place l % kPieces, and the
+    // hardware puts the lanes' 16 bytes side by side.
     // The caller's arrays are readable up to the next multiple of kRowPad
     // rows, and a row is a whole number of chunks: no clamping
     const int my_first = wave * kWaveRows;      // among the BM + BN rows of a buffer
     const bool brings_query = my_first < BM;
     const int bring_row = lane / kPieces;
     const unsigned bring_off =
-        ((unsigned)((brings_query ? my_first : my_first - BM) + bring_row) * (unsigned)a.d) * 2u +
-        16u * ((lane % kPieces) ^ ((bring_row / (8 / kPieces)) & (kPieces - 1)));
+        ((unsigned)((brings_query ? my_first : my_first - BM) + bring_row) * (unsigned)a.d) * 2u;
     const unsigned char *a_base =
         reinterpret_cast<const unsigned char *>(a.query) + (size_t)q0 * a.d * 2;
     const unsigned bring_to =
         (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)stage + my_first * kRow;
     // operand reads: lane l wants elements 16 s + 8 (l / 32) .. + 8 of row
     // l % 32 of an instruction tile, piece 2 s + l / 32 of that row
-    const unsigned mix = (col / (8 / kPieces)) & (kPieces - 1);
+    const unsigned mix = PA_PLACE_MIX(col);
     const unsigned swizzle = 16u * (half ^ (mix & 1)) + 32u * (mix >> 1);
     const unsigned char *a_tile = stage + (wr * WM * 32 + col) * kRow;
     const unsigned char *b_tile = stage + (BM + wc * WN * 32 + col) * kRow;
@@ -232,7 +235,8 @@ __global__ __launch_bounds__(64 * WR * WC, (WM * WN > 8 ? 1 : 2)) void knn_kerne
                               : reinterpret_cast<const unsigned char *>(a.base) +       \
                                     ((size_t)f_tile * BN * a.d + f_k0) * 2) + bring_off;\
             _Pragma("unroll") for (int i = 0; i < kInstrs; ++i)                         \
-                bring_rows(from + (size_t)(kInstrRows * i) * a.d * 2,                   \
+                bring_rows(from + (size_t)(kInstrRows * i) * a.d * 2 +                  \
+                               16u * ((lane % kPieces) ^ PA_PLACE_MIX(kInstrRows * i + bring_row)), \
                            bring_to + (buf) * kStage + kInstrRows * i * kRow);          \
             f_k0 += kChunk;                                                             \
             if (f_k0 >= a.d) f_k0 = 0, f_tile += a.n_seg;                               \
@@ -346,6 +350,7 @@ __global__ __launch_bounds__(64 * WR * WC, (WM * WN > 8 ? 1 : 2)) void knn_kerne
         // counts and limits again
     }
 #undef PA_FETCH_NEXT
+#undef PA_PLACE_MIX
 #undef PA_LOAD_NORMS
     __syncthreads();
     {
