@@ -36,7 +36,6 @@ namespace {
 
 typedef _Float16 half8 __attribute__((ext_vector_type(8)));
 typedef float floatx16 __attribute__((ext_vector_type(16)));
-typedef unsigned int uintx4 __attribute__((ext_vector_type(4)));
 
 constexpr int kChunk = 64;        // contraction elements staged at a time; a
                                   // row is a whole number of chunks
