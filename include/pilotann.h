@@ -263,6 +263,18 @@ int pa_knn(float *cand_score, int32_t *cand_id, int32_t *cand_count,
            int64_t m, int64_t n, int d, int keep, int n_seg, void *stream);
 
 /*
+ * The exact ranking that follows pa_knn (faiss' part in the reference,
+ * pilot_ann/utils/graphs.py:15-20; no entry point of the reference's extension
+ * corresponds to it): dist [m * k] receives the squared float32 distances
+ * from rows first .. first + m of `rows` [n * d] to their candidates
+ * cand [m * k] (int64 row numbers); infinity for a candidate that is -1, out
+ * of range or the row itself.  d % 4 == 0, d <= 4096.  Device pointers;
+ * enqueued on `stream`.
+ */
+int pa_knn_rerank(float *dist, const float *rows, const int64_t *cand,
+                  int64_t m, int64_t first, int64_t n, int d, int k, void *stream);
+
+/*
  * Occlusion pruning of candidate lists, the edge selection of the graph
  * builder (faiss' part in the reference, pilot_ann/utils/graphs.py:15-20,52-56;
  * no entry point of the reference's extension corresponds to it).  For each of

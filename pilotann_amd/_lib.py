@@ -37,6 +37,7 @@ _SIGNATURES = {
                                   _int, _int, _int, _int]),
     'pa_knn_list_capacity': (_i64, [_int]),
     'pa_knn_tile_rows': (_int, []),
+    'pa_knn_rerank': (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _int, _vp]),
     'pa_knn': (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _int, _vp]),
     'pa_graph_prune': (_int, [_vp, _vp, _vp, _i64, _int, _int, _int, _vp]),
     'pa_heapq_pop': (_int, [_vp, _vp, _i64]),

@@ -368,6 +368,51 @@ __global__ __launch_bounds__(64 * WR * WC, (WM * WN > 8 ? 1 : 2)) void knn_kerne
         if (q0 + r < a.m) a.cand_count[(size_t)seg * a.m + q0 + r] = count[r];
 }
 
+// Exact squared distances from query row first + q to its candidates, the
+// float arithmetic of the search itself (differences, then squares, summed).
+// A wavefront per query, its row in LDS; 16 lanes per candidate, four
+// candidates at a time, every lane 16 bytes of the candidate's row per step.
+// A candidate that is -1, out of range or the query row itself gets infinity.
+constexpr int kRankWaves = 4;
+
+__global__ __launch_bounds__(kWave * kRankWaves) void rerank_kernel(
+    const float *__restrict__ rows, const int64_t *__restrict__ cand,
+    float *__restrict__ out, int64_t m, int64_t first, int64_t n, int d, int k) {
+    typedef float floatx4 __attribute__((ext_vector_type(4)));
+    extern __shared__ __align__(16) unsigned char rank_lds[];
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    const int64_t q = (int64_t)blockIdx.x * kRankWaves + wave;
+    const int d4 = d / 4;
+    floatx4 *mine = reinterpret_cast<floatx4 *>(rank_lds) + wave * d4;
+    if (q < m) {
+        const floatx4 *src = reinterpret_cast<const floatx4 *>(rows + (size_t)(first + q) * d);
+        for (int i = lane; i < d4; i += kWave) mine[i] = src[i];
+    }
+    __syncthreads();
+    if (q >= m) return;
+    const int team = lane >> 4, place = lane & 15;
+    for (int j0 = 0; j0 < k; j0 += 4) {
+        const int j = j0 + team;
+        const int64_t id = j < k ? cand[(size_t)q * k + j] : -1;
+        const bool ok = id >= 0 && id < n && id != first + q;
+        float sum = 0.f;
+        if (ok) {
+            const floatx4 *row = reinterpret_cast<const floatx4 *>(rows + (size_t)id * d);
+            for (int i = place; i < d4; i += 16) {
+                const floatx4 x = row[i], y = mine[i];
+                const float e0 = x[0] - y[0], e1 = x[1] - y[1], e2 = x[2] - y[2], e3 = x[3] - y[3];
+                sum = fmaf(e0, e0, sum);
+                sum = fmaf(e1, e1, sum);
+                sum = fmaf(e2, e2, sum);
+                sum = fmaf(e3, e3, sum);
+            }
+        }
+#pragma unroll
+        for (int step = 8; step >= 1; step >>= 1) sum += __shfl_xor(sum, step, 16);
+        if (place == 0 && j < k) out[(size_t)q * k + j] = ok ? sum : INFINITY;
+    }
+}
+
 // Occlusion pruning of a node's candidate list (closest first): candidate j
 // is kept unless a candidate kept before it is closer to it than the node
 // itself is, until m_keep are kept; with `fill` the closest rejected ones top
@@ -466,6 +511,20 @@ extern "C" int pa_knn(float *cand_score, int32_t *cand_id, int32_t *cand_count,
         case 256: return launch_knn<256>(a, stream);
         default: return launch_knn<512>(a, stream);
     }
+}
+
+extern "C" int pa_knn_rerank(float *dist, const float *rows, const int64_t *cand,
+                             int64_t m, int64_t first, int64_t n, int d, int k,
+                             void *stream_) {
+    if (m < 0 || n < 0 || first < 0 || first + m > n || k < 1) return PA_E_SHAPE;
+    if (d <= 0 || d % 4 || d > 4096) return PA_E_DIM;
+    if ((m + kRankWaves - 1) / kRankWaves >= (1ll << 31)) return PA_E_RANGE;
+    if (m == 0) return PA_OK;
+    if (!dist || !rows || !cand) return PA_E_NULL;
+    const unsigned lds = (unsigned)(kRankWaves * d * sizeof(float));
+    rerank_kernel<<<(unsigned)((m + kRankWaves - 1) / kRankWaves), kWave * kRankWaves, lds,
+                    (hipStream_t)stream_>>>(rows, cand, dist, m, first, n, d, k);
+    return (int)hipGetLastError();
 }
 
 extern "C" int pa_graph_prune(int32_t *selected, const float *pair,

@@ -379,6 +379,25 @@ def knn_candidates(query, base, keep: int, n_seg: int = None):
     return torch.gather(ids, 1, top.indices)
 
 
+def knn_rerank(rows: torch.Tensor, cand: torch.Tensor, first: int = 0):
+    """Exact squared float32 distances ``[m, k]`` from rows ``first ..
+    first + m`` of ``rows`` to their candidates ``cand`` ``[m, k]`` (int64 row
+    numbers; ``pa_knn_rerank``): infinity where a candidate is ``-1`` or the
+    row itself.  The ranking step after :func:`knn_candidates`."""
+    _check(rows, 'rows', 2, torch.float32, True)
+    _check(cand, 'cand', 2, torch.int64, True)
+    _require(cand.device == rows.device, 'cand.device == rows.device')
+    m, k = cand.shape
+    n, d = rows.shape
+    _require(0 <= first and first + m <= n, 'first + cand.size(0) <= rows.size(0)')
+    dist = torch.empty(m, k, dtype=torch.float32, device=rows.device)
+    with torch.cuda.device(rows.device):
+        _lib.check(_lib.lib().pa_knn_rerank(
+            _ptr(dist), _ptr(rows), _ptr(cand), m, int(first), n, d, k, _stream()),
+            'pa_knn_rerank')
+    return dist
+
+
 def graph_prune(pair: torch.Tensor, cand_dist: torch.Tensor, m_keep: int, fill: bool):
     """Occlusion pruning of candidate lists (``pa_graph_prune``): ``pair``
     ``[n, k, k]`` distances between a node's candidates, ``cand_dist``

@@ -64,13 +64,24 @@ def _knn_graph_device(x: torch.Tensor, k: int, rows_per_pass: int = None):
     rows = kernels.HalfRows(x)
     out_i = torch.empty(n, k, dtype=torch.long, device=x.device)
     out_d = torch.empty(n, k, dtype=torch.float32, device=x.device)
-    # candidate lists of a pass: 2 * (keep + 256) * 4 bytes a row
+    # candidate lists of a pass: 2 * (keep + 384) * 4 bytes a row
     pass_rows = 1 << 21
+    fused = d % 4 == 0 and d <= 4096 and rows_per_pass is None
     if rows_per_pass is None:
         rows_per_pass = max(256, min(8192, (1 << 29) // (keep * d)))
     for lo in range(0, n, pass_rows):
         hi = min(n, lo + pass_rows)
         cand = kernels.knn_candidates(rows.rows(lo, hi), rows, keep)
+        if fused:
+            # exact distances to the candidates by one kernel
+            d2 = kernels.knn_rerank(x, cand, lo)
+            top = torch.topk(d2, k, dim=-1, largest=False)
+            out_i[lo:hi] = torch.gather(cand, 1, top.indices)
+            out_d[lo:hi] = top.values
+            del d2
+            if progress is not None:
+                progress(f'neighbour table: {hi} of {n} rows')
+            continue
         own = torch.arange(lo, hi, device=x.device).unsqueeze(-1)
         for a in range(0, hi - lo, rows_per_pass):
             b = min(hi - lo, a + rows_per_pass)

@@ -30,7 +30,7 @@ def overlap(got, want):
 @pytest.mark.parametrize('n,d,k', [
     (129, 8, 5), (1000, 64, 10), (5000, 72, 47), (5000, 72, 48),
     (20000, 96, 64), (3000, 200, 111), (3000, 200, 127), (12345, 768, 80),
-    (9000, 64, 240), (3000, 128, 496), (3000, 128, 497),
+    (9000, 64, 240), (3000, 128, 496), (3000, 128, 497), (2000, 192, 20), (700, 50, 9),
 ])
 def test_knn_table_is_the_exact_one(n, d, k, device):
     print('knn case', n, d, k, flush=True)
@@ -103,6 +103,28 @@ def test_a_part_of_a_prepared_set_as_queries(device):
     assert overlap(part, want) > 0.9995
     with pytest.raises(RuntimeError):
         rows.rows(100, 3000)
+
+
+@pytest.mark.parametrize('n,d,m,k,first', [(500, 4, 500, 7, 0), (3000, 768, 1000, 256, 512),
+                                           (2000, 100, 333, 65, 1667), (300, 4096, 5, 3, 295)])
+def test_exact_distances_to_candidates(n, d, m, k, first, device):
+    """pa_knn_rerank: float32 distances from rows first .. first + m to their
+    candidates, infinity for -1 and for the row itself."""
+    print('knn rerank', n, d, m, k, first, flush=True)
+    g = torch.Generator().manual_seed(n + d)
+    x = torch.randn(n, d, generator=g)
+    cand = torch.randint(0, n, (m, k), generator=g)
+    cand[::3, 0] = -1
+    cand[1::3, -1] = torch.arange(first, first + m)[1::3]          # the row itself
+    got = kernels.knn_rerank(x.to(device), cand.to(device), first).cpu()
+    want = (x[cand.clamp(min=0)].double() - x[first:first + m].double().unsqueeze(1)).square().sum(-1)
+    skip = (cand < 0) | (cand == torch.arange(first, first + m).unsqueeze(1))
+    assert bool(torch.isinf(got[skip]).all()) and bool((got[skip] > 0).all())
+    assert torch.allclose(got[~skip].double(), want[~skip], rtol=2e-6, atol=0)
+    with pytest.raises(RuntimeError):
+        kernels.knn_rerank(x.to(device), cand.to(device), n - m + 1)
+    with pytest.raises(RuntimeError):
+        kernels.knn_rerank(x[:, :3].contiguous().to(device), cand.to(device), first)
 
 
 def test_fewer_base_rows_than_candidates(device):
