@@ -597,7 +597,8 @@ def main():
     if args.full_index:
         cfg['stage_only'] = False
         from pilotann_amd.utils import graphs
-        graphs.progress = lambda text: log('[bench] ' + text)
+        started = time.time()
+        graphs.progress = lambda text: log(f'[bench] {time.time() - started:6.1f}s {text}')
     if args.stage_cache and not cfg.get('stage_only'):
         ap.error('--stage-cache is for configurations that build the device '
                  'stage only')

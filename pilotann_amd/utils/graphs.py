@@ -80,6 +80,7 @@ def _knn_graph_device(x: torch.Tensor, k: int, rows_per_pass: int = None):
             out_d[lo:hi] = top.values
             del d2
             if progress is not None:
+                torch.cuda.synchronize(x.device)   # report what is done, not what is queued
                 progress(f'neighbour table: {hi} of {n} rows')
             continue
         own = torch.arange(lo, hi, device=x.device).unsqueeze(-1)
@@ -108,12 +109,16 @@ def _occlusion_prune(x, cand, cand_d, m_keep: int, fill: bool, chunk: int):
     on_device = x.is_cuda and K <= 512
     if on_device:
         from .. import kernels
+    norms = x.float().square().sum(-1)
     for lo in range(0, n, chunk):
+        if progress is not None and (lo // chunk) % 512 == 511:
+            progress(f'pruning: {lo} of {n} rows')
         c = cand[lo:lo + chunk]
         cd = cand_d[lo:lo + chunk]
         v = x[c].float()
-        sq = v.square().sum(-1)
-        pair = sq.unsqueeze(-1) + sq.unsqueeze(-2) - 2.0 * (v @ v.mT)
+        sq = norms[c]
+        # |a|^2 + |b|^2 - 2 a.b in one pass over the products
+        pair = torch.baddbmm(sq.unsqueeze(-1) + sq.unsqueeze(-2), v, v.mT, alpha=-2.0)
         del v
         if on_device:
             # the greedy pass over the candidates, one wavefront per node
@@ -245,6 +250,8 @@ def connect_graph(x: torch.Tensor, adj: torch.Tensor, hub: int = None,
         if bool(ok.all()):
             return round_
         cut = torch.nonzero(~ok).flatten()
+        if progress is not None:
+            progress(f'connectivity: round {round_}, {cut.numel()} of {n} nodes cut off')
         if cut.numel() > per_round:
             pick = torch.randperm(cut.numel(), generator=g)[:per_round]
             cut = cut[pick.to(dev)]
