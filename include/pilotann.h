@@ -289,6 +289,25 @@ int pa_graph_prune(int32_t *selected, const float *pair, const float *cand_dist,
                    int64_t n, int k, int m_keep, int fill, void *stream);
 
 /*
+ * The same pruning straight from the rows (no counterpart in the reference's
+ * extension either): the distances between a node's k <= 256 candidates are
+ * made inside the kernel and never stored.  rows_hi_f16 / rows_lo_f16 hold
+ * every row as two half-precision parts (row * s = hi + lo, rows of d
+ * elements, d % 64 == 0, padded with zeros), norm [rows] the squared lengths
+ * of the scaled rows, cand [n * k] the candidates' row numbers (closest first,
+ * -1 after the last), cand_dist [n * k] their squared distances to the node in
+ * the rows' own units and scale2 = s * s.  A pair's distance is
+ * |a|^2 + |b|^2 - 2 (hi.hi + hi.lo + lo.hi): the float32 value to about 22
+ * bits.  selected as for pa_graph_prune.  Device pointers; enqueued on
+ * `stream`.
+ */
+int pa_graph_prune_rows(int32_t *selected, const void *rows_hi_f16,
+                        const void *rows_lo_f16, const float *norm,
+                        const int64_t *cand, const float *cand_dist, int64_t n,
+                        int d, int k, int m_keep, int fill, float scale2,
+                        void *stream);
+
+/*
  * The reference's operator hooks (extension/ops_cpu.cpp:8-95,
  * pilot_ann/kernels/__init__.py:5-35): one call of a heap primitive of
  * extension/inc/heapq.cuh on a host array heap of n (key, value) cells, a set

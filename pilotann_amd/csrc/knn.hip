@@ -465,6 +465,188 @@ __global__ __launch_bounds__(256) void prune_kernel(
     for (int i = count + lane; i < m_keep; i += kWave) out[i] = -1;
 }
 
+// Occlusion pruning straight from the rows: the same rule as prune_kernel,
+// with the candidate-to-candidate distances made on the spot.  A workgroup of
+// eight wavefronts takes one node: it gathers the rows of the node's k <= 256
+// candidates chunk by chunk into LDS (the transfers of knn_kernel, every lane
+// with the address of its own candidate's row), multiplies them with
+// themselves on the matrix cores — rows as two half-precision parts, x = hi +
+// lo, and hi.hi + hi.lo + lo.hi for the product, which is the float product to
+// about 22 bits — and reduces |a|^2 + |b|^2 - 2 a.b < dist(node, a) to one bit
+// per pair in LDS; then its first wavefront walks the candidates in order
+// against the bits of those kept so far.  The k x k table never leaves the CU.
+struct PruneRowsArgs {
+    const _Float16 *hi, *lo;
+    const float *norm;        // squared lengths of the scaled rows
+    const int64_t *cand;      // [n, k] row numbers, closest first, -1 after the last
+    const float *cand_dist;   // [n, k] squared distances to the node, unscaled
+    int32_t *selected;        // [n, m_keep]
+    int64_t n;
+    int d, k, m_keep, fill;
+    float scale2;             // (scaled / unscaled) squared
+};
+
+__global__ __launch_bounds__(512, 2) void prune_rows_kernel(PruneRowsArgs a) {
+    constexpr int kRows = 256;                 // candidates of a node, padded
+    constexpr int kRow = kChunk * 2;           // bytes of a staged row
+    constexpr int kPart = kRows * kRow;        // one part (hi or lo) of a chunk
+    constexpr int kStage = 2 * kPart;
+    constexpr int kWords = kRows / 32;
+    __shared__ __align__(1024) unsigned char stage[2 * kStage];
+    __shared__ unsigned bits[kRows][kWords];   // bits[a][w]: bit b % 32 of word b / 32 says b blocks a
+    __shared__ float len2[kRows], reach[kRows];
+    __shared__ int valid_count;
+    const int t = threadIdx.x;
+    const int lane = t & (kWave - 1), wave = t / kWave;
+    const int wr = wave % 2, wc = wave / 2;
+    const int col = lane & 31, half = lane >> 5;
+    const int64_t node = blockIdx.x;
+    const int64_t *ids = a.cand + (size_t)node * a.k;
+
+    // the candidates' lengths and distances; what lies behind the list
+    // repeats the first candidate and can block nothing
+    if (t < kRows) {
+        const int64_t id = t < a.k ? ids[t] : -1;
+        len2[t] = id >= 0 ? a.norm[id] : 0.f;
+        reach[t] = id >= 0 ? a.cand_dist[(size_t)node * a.k + t] * a.scale2 : -INFINITY;
+    }
+    if (t == 0) valid_count = 0;
+    __syncthreads();
+    if (t < a.k && ids[t] >= 0) atomicAdd(&valid_count, 1);
+
+    // transfers: wavefront w brings rows 32 w .. 32 w + 31 of both parts, 8
+    // rows an instruction, lane l the piece that belongs at place l % 8 of row
+    // l / 8 (places as in knn_kernel)
+    const int bring_row = lane >> 3;
+    size_t from[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = 32 * wave + 8 * i + bring_row;
+        int64_t id = row < a.k ? ids[row] : -1;
+        if (id < 0) id = ids[0] >= 0 ? ids[0] : 0;
+        from[i] = ((size_t)id * a.d) * 2 + 16u * ((lane & 7) ^ (((8 * i + bring_row) >> 1) & 7));
+    }
+    const unsigned bring_to =
+        (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char *)stage +
+        32 * wave * kRow;
+    const unsigned char *hi = reinterpret_cast<const unsigned char *>(a.hi);
+    const unsigned char *lo = reinterpret_cast<const unsigned char *>(a.lo);
+#define PA_BRING_CHUNK(k0, buf)                                                          \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                      \
+        bring_rows(hi + from[i] + (size_t)(k0) * 2, bring_to + (buf) * kStage + 8 * i * kRow); \
+        bring_rows(lo + from[i] + (size_t)(k0) * 2,                                      \
+                   bring_to + (buf) * kStage + kPart + 8 * i * kRow);                    \
+    }
+    const unsigned mix = (col >> 1) & 7;
+    const unsigned swizzle = 16u * (half ^ (mix & 1)) + 32u * (mix >> 1);
+    const unsigned char *a_tile = stage + (wr * 128 + col) * kRow;
+    const unsigned char *b_tile = stage + (wc * 64 + col) * kRow;
+
+    floatx16 acc[4][2];
+#pragma unroll
+    for (int m = 0; m < 4; ++m)
+#pragma unroll
+        for (int n = 0; n < 2; ++n)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[m][n][r] = 0.f;
+
+    PA_BRING_CHUNK(0, 0)
+    bring_wait<0>();
+    __syncthreads();
+    int buf = 0;
+#pragma unroll 1
+    for (int k0 = 0; k0 < a.d; k0 += kChunk, buf ^= 1) {
+        if (k0 + kChunk < a.d) PA_BRING_CHUNK(k0 + kChunk, buf ^ 1)
+        const unsigned char *a_now = a_tile + buf * kStage, *b_now = b_tile + buf * kStage;
+#pragma unroll
+        for (int s = 0; s < kChunk / 16; ++s) {
+            const unsigned at = swizzle ^ (32u * s);
+            half8 av[4], bv[2];
+            // hi . hi
+#pragma unroll
+            for (int m = 0; m < 4; ++m)
+                av[m] = *reinterpret_cast<const half8 *>(a_now + m * 32 * kRow + at);
+#pragma unroll
+            for (int n = 0; n < 2; ++n)
+                bv[n] = *reinterpret_cast<const half8 *>(b_now + n * 32 * kRow + at);
+#pragma unroll
+            for (int m = 0; m < 4; ++m)
+#pragma unroll
+                for (int n = 0; n < 2; ++n)
+                    acc[m][n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[m], bv[n], acc[m][n], 0, 0, 0);
+            // hi . lo
+#pragma unroll
+            for (int n = 0; n < 2; ++n)
+                bv[n] = *reinterpret_cast<const half8 *>(b_now + kPart + n * 32 * kRow + at);
+#pragma unroll
+            for (int m = 0; m < 4; ++m)
+#pragma unroll
+                for (int n = 0; n < 2; ++n)
+                    acc[m][n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[m], bv[n], acc[m][n], 0, 0, 0);
+            // lo . hi
+#pragma unroll
+            for (int m = 0; m < 4; ++m)
+                av[m] = *reinterpret_cast<const half8 *>(a_now + kPart + m * 32 * kRow + at);
+#pragma unroll
+            for (int n = 0; n < 2; ++n)
+                bv[n] = *reinterpret_cast<const half8 *>(b_now + n * 32 * kRow + at);
+#pragma unroll
+            for (int m = 0; m < 4; ++m)
+#pragma unroll
+                for (int n = 0; n < 2; ++n)
+                    acc[m][n] = __builtin_amdgcn_mfma_f32_32x32x16_f16(av[m], bv[n], acc[m][n], 0, 0, 0);
+        }
+        bring_wait<0>();
+        __syncthreads();
+    }
+#undef PA_BRING_CHUNK
+
+    // a lane's 16 results of an instruction tile are
+    // D[i = 8 * (r / 4) + 4 * (l / 32) + r % 4][j = l % 32]: one ballot is the
+    // word of 32 columns for two rows
+#pragma unroll
+    for (int n = 0; n < 2; ++n) {
+        const int b = (wc * 2 + n) * 32 + col;
+        const float len_b = len2[b];
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = (wr * 4 + m) * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+                const float pair = (len2[row] + len_b) - 2.f * acc[m][n][r];
+                const unsigned long long word = __ballot(pair < reach[row]);
+                if (col == 0)
+                    bits[row][wc * 2 + n] = half ? (unsigned)(word >> 32) : (unsigned)word;
+            }
+        }
+    }
+    __syncthreads();
+    if (wave != 0) return;
+
+    // the walk: lane w < 8 holds word w of the kept set
+    int32_t *out = a.selected + (size_t)node * a.m_keep;
+    const int k_valid = valid_count;
+    unsigned kept = 0;
+    int count = 0;
+    for (int j = 0; j < k_valid && count < a.m_keep; ++j) {
+        const unsigned hit = lane < kWords ? (bits[j][lane] & kept) : 0u;
+        if (!__ballot(hit != 0)) {
+            if (lane == (j >> 5)) kept |= 1u << (j & 31);
+            if (lane == 0) out[count] = j;
+            count += 1;
+        }
+    }
+    if (a.fill) {
+        for (int j = 0; j < k_valid && count < a.m_keep; ++j) {
+            const unsigned word = __builtin_amdgcn_readlane(kept, j >> 5);
+            if ((word >> (j & 31)) & 1u) continue;
+            if (lane == 0) out[count] = j;
+            count += 1;
+        }
+    }
+    for (int i = count + lane; i < a.m_keep; i += kWave) out[i] = -1;
+}
+
 // The form in use: 2 x 4 wavefronts of 4 x 2 instruction tiles, 256 query rows
 // against 256 base rows per tile; one workgroup per compute unit (150 KB of
 // LDS, 256 registers a lane).
@@ -524,6 +706,26 @@ extern "C" int pa_knn_rerank(float *dist, const float *rows, const int64_t *cand
     const unsigned lds = (unsigned)(kRankWaves * d * sizeof(float));
     rerank_kernel<<<(unsigned)((m + kRankWaves - 1) / kRankWaves), kWave * kRankWaves, lds,
                     (hipStream_t)stream_>>>(rows, cand, dist, m, first, n, d, k);
+    return (int)hipGetLastError();
+}
+
+extern "C" int pa_graph_prune_rows(int32_t *selected, const void *rows_hi_f16,
+                                   const void *rows_lo_f16, const float *norm,
+                                   const int64_t *cand, const float *cand_dist,
+                                   int64_t n, int d, int k, int m_keep, int fill,
+                                   float scale2, void *stream_) {
+    if (n < 0 || k < 1 || k > 256 || m_keep < 1) return PA_E_SHAPE;
+    if (d <= 0 || d % kChunk) return PA_E_DIM;
+    if (n >= (1ll << 31)) return PA_E_RANGE;
+    if (n == 0) return PA_OK;
+    if (!selected || !rows_hi_f16 || !rows_lo_f16 || !norm || !cand || !cand_dist)
+        return PA_E_NULL;
+    PruneRowsArgs a;
+    a.hi = reinterpret_cast<const _Float16 *>(rows_hi_f16);
+    a.lo = reinterpret_cast<const _Float16 *>(rows_lo_f16);
+    a.norm = norm, a.cand = cand, a.cand_dist = cand_dist, a.selected = selected;
+    a.n = n, a.d = d, a.k = k, a.m_keep = m_keep, a.fill = fill, a.scale2 = scale2;
+    prune_rows_kernel<<<(unsigned)n, 512, 0, (hipStream_t)stream_>>>(a);
     return (int)hipGetLastError();
 }
 

@@ -319,6 +319,14 @@ class HalfRows:
         self.norm = torch.zeros(n_pad, dtype=torch.float32, device=rows.device)
         self.norm[:n] = (rows * scale).square().sum(-1)
 
+    def low(self, rows: torch.Tensor) -> torch.Tensor:
+        """The second half-precision part of ``rows`` (the tensor this set was
+        made from): ``rows * scale - half``, same shape and padding as
+        ``half``, so that ``half + low`` is the scaled row to about 22 bits."""
+        low = torch.zeros_like(self.half)
+        low[:self.n, :self.d] = rows * self.scale - self.half[:self.n, :self.d].float()
+        return low
+
     def rows(self, lo: int, hi: int) -> 'HalfRows':
         """Rows ``lo .. hi`` as a set of their own (a view; ``lo`` a multiple
         of the tile, so that the padding still reaches a whole tile)."""
@@ -413,6 +421,32 @@ def graph_prune(pair: torch.Tensor, cand_dist: torch.Tensor, m_keep: int, fill: 
         _lib.check(_lib.lib().pa_graph_prune(
             _ptr(selected), _ptr(pair), _ptr(cand_dist), n, k, int(m_keep),
             int(bool(fill)), _stream()), 'pa_graph_prune')
+    return selected.long()
+
+
+def graph_prune_rows(rows: torch.Tensor, cand: torch.Tensor, cand_dist: torch.Tensor,
+                     m_keep: int, fill: bool):
+    """:func:`graph_prune` without the table of pairwise distances
+    (``pa_graph_prune_rows``): ``rows`` ``[N, d]`` float32, ``cand`` ``[n, k]``
+    int64 row numbers (closest first, ``-1`` after the last, ``k <= 256``),
+    ``cand_dist`` ``[n, k]`` their squared distances to the node.  Returns the
+    positions ``[n, m_keep]`` as :func:`graph_prune` does."""
+    _check(rows, 'rows', 2, torch.float32, True)
+    _check(cand, 'cand', 2, torch.int64, True)
+    _check(cand_dist, 'cand_dist', 2, torch.float32, True)
+    _require(cand.shape == cand_dist.shape, 'cand.shape == cand_dist.shape')
+    _require(cand.device == rows.device == cand_dist.device, 'one device')
+    n, k = cand.shape
+    _require(1 <= k <= 256, '1 <= k <= 256')
+    _require(int(cand.max()) < rows.size(0), 'cand < rows.size(0)')
+    parts = HalfRows(rows)
+    low = parts.low(rows)
+    selected = torch.empty(n, int(m_keep), dtype=torch.int32, device=rows.device)
+    with torch.cuda.device(rows.device):
+        _lib.check(_lib.lib().pa_graph_prune_rows(
+            _ptr(selected), _ptr(parts.half), _ptr(low), _ptr(parts.norm), _ptr(cand),
+            _ptr(cand_dist), n, parts.half.size(1), k, int(m_keep), int(bool(fill)),
+            float(parts.scale) ** 2, _stream()), 'pa_graph_prune_rows')
     return selected.long()
 
 

@@ -18,6 +18,9 @@ import torch
 # (a pass of the neighbour kernel over two million rows, say): a caller that
 # must show signs of life sets it (``graphs.progress = print``).
 progress = None
+# the pruning of the builder in one kernel (``kernels.graph_prune_rows``); off:
+# gathered rows, a batched product of torch and ``kernels.graph_prune``
+fused_prune = True
 
 
 def knn_graph(x: torch.Tensor, k: int, chunk: int = None,
@@ -109,6 +112,13 @@ def _occlusion_prune(x, cand, cand_d, m_keep: int, fill: bool, chunk: int):
     on_device = x.is_cuda and K <= 512
     if on_device:
         from .. import kernels
+    if on_device and K <= 256 and x.dtype == torch.float32 and fused_prune:
+        # gather, pairwise distances and the greedy pass in one kernel
+        sel = kernels.graph_prune_rows(x.contiguous(), cand.contiguous(),
+                                       cand_d.float().contiguous(), min(m_keep, K), fill)
+        ids = torch.gather(cand, 1, sel.clamp(min=0))
+        out[:, :ids.size(1)] = torch.where(sel >= 0, ids, torch.full_like(ids, -1))
+        return out
     norms = x.float().square().sum(-1)
     for lo in range(0, n, chunk):
         if progress is not None and (lo // chunk) % 512 == 511:

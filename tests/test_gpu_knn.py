@@ -209,3 +209,45 @@ def test_occlusion_pruning_equals_the_step_by_step_rule(n, k, m_keep, fill, devi
     assert torch.equal(got, want)
     with pytest.raises(RuntimeError):
         kernels.graph_prune(pair[:, :, :-1].contiguous().to(device), d.to(device), m_keep, fill)
+
+
+@pytest.mark.parametrize('n,d,k,m_keep,fill', [
+    (3000, 64, 240, 32, True), (2000, 768, 240, 48, False), (1500, 100, 64, 16, True),
+    (400, 128, 256, 32, True), (40, 64, 39, 32, True), (300, 192, 9, 4, False),
+])
+def test_pruning_straight_from_the_rows(n, d, k, m_keep, fill, device):
+    """`pa_graph_prune_rows` against `pa_graph_prune` on the float32 table of
+    pairwise distances: the same selection, except where a pair's distance and
+    the candidate's own differ by less than the two-part products resolve."""
+    print('prune rows case', n, d, k, m_keep, fill, flush=True)
+    x = utils.gaussian_mixture(n, d, 8, 1.0, seed=n + d, decay=0.3).to(device)
+    cand, cand_d = utils.knn_graph(x, k)
+    if k == 39:                                   # lists that end in -1
+        cand[::2, -5:] = -1
+        cand_d[::2, -5:] = float('inf')
+    got = kernels.graph_prune_rows(x, cand, cand_d, m_keep, fill)
+    v = x[cand.clamp(min=0)].double()
+    sq = v.square().sum(-1)                        # float64: the product form is exact enough
+    pair = (sq.unsqueeze(-1) + sq.unsqueeze(-2) - 2.0 * (v @ v.mT)).clamp_(min=0.0)
+    valid = cand >= 0
+    pair[~(valid.unsqueeze(2) & valid.unsqueeze(1))] = float('inf')
+    want = kernels.graph_prune(pair.float().contiguous(), cand_d.contiguous(), m_keep, fill)
+    if k == 39:
+        # candidates behind the end of a list do not exist for the kernel:
+        # those rows against the pruning of their first 34 candidates
+        short = kernels.graph_prune(pair[::2, :34, :34].float().contiguous(),
+                                    cand_d[::2, :34].contiguous(), m_keep, fill)
+        want[::2] = short
+    same = (got == want).all(-1)
+    torch.cuda.synchronize()
+    assert int(got.max()) < k and int(got.min()) >= -1
+    assert float(same.float().mean()) > 0.995, float(same.float().mean())
+    # a row that differs does so at a near-tie
+    margin = ((pair - cand_d.double().unsqueeze(-1)).abs() /
+              cand_d.double().unsqueeze(-1).clamp(min=1e-30))
+    margin[~(valid.unsqueeze(2) & valid.unsqueeze(1))] = float('inf')
+    tight = margin.flatten(1).min(-1).values
+    assert bool((tight[~same] < 1e-4).all())
+    with pytest.raises(RuntimeError):
+        kernels.graph_prune_rows(x, cand[:, :1].expand(-1, 300).contiguous(),
+                                 cand_d[:, :1].expand(-1, 300).contiguous(), m_keep, fill)
