@@ -475,13 +475,15 @@ __global__ __launch_bounds__(256) void prune_kernel(
 // about 22 bits — and reduces |a|^2 + |b|^2 - 2 a.b < dist(node, a) to one bit
 // per pair in LDS; then its first wavefront walks the candidates in order
 // against the bits of those kept so far.  The k x k table never leaves the CU.
+constexpr int64_t kLaunchNodes = 1ll << 22;
+
 struct PruneRowsArgs {
     const _Float16 *hi, *lo;
     const float *norm;        // squared lengths of the scaled rows
     const int64_t *cand;      // [n, k] row numbers, closest first, -1 after the last
     const float *cand_dist;   // [n, k] squared distances to the node, unscaled
     int32_t *selected;        // [n, m_keep]
-    int64_t n;
+    int64_t n, first;         // this launch takes nodes first .. first + gridDim.x
     int d, k, m_keep, fill;
     float scale2;             // (scaled / unscaled) squared
 };
@@ -500,7 +502,7 @@ __global__ __launch_bounds__(512, 2) void prune_rows_kernel(PruneRowsArgs a) {
     const int lane = t & (kWave - 1), wave = t / kWave;
     const int wr = wave % 2, wc = wave / 2;
     const int col = lane & 31, half = lane >> 5;
-    const int64_t node = blockIdx.x;
+    const int64_t node = a.first + blockIdx.x;
     const int64_t *ids = a.cand + (size_t)node * a.k;
 
     // the candidates' lengths and distances; what lies behind the list
@@ -673,7 +675,9 @@ extern "C" int pa_knn(float *cand_score, int32_t *cand_id, int32_t *cand_count,
                       const float *base_norm, int64_t m, int64_t n, int d,
                       int keep, int n_seg, void *stream_) {
     if (m < 0 || n < 0 || n_seg < 1 || n_seg > 65535) return PA_E_SHAPE;
-    if (n >= (1ll << 31) || (m + kBM - 1) / kBM >= (1ll << 31)) return PA_E_RANGE;
+    // ids are 32 bits, and a launch holds fewer than 2^32 work-items
+    if (n >= (1ll << 31) || (m + kBM - 1) / kBM * n_seg >= (1ll << 32) / (64 * kWR * kWC))
+        return PA_E_RANGE;
     if (d <= 0 || d % kChunk) return PA_E_DIM;
     if (keep != 64 && keep != 128 && keep != 256 && keep != 512) return PA_E_SHAPE;
     if (m == 0) return PA_OK;
@@ -700,7 +704,7 @@ extern "C" int pa_knn_rerank(float *dist, const float *rows, const int64_t *cand
                              void *stream_) {
     if (m < 0 || n < 0 || first < 0 || first + m > n || k < 1) return PA_E_SHAPE;
     if (d <= 0 || d % 4 || d > 4096) return PA_E_DIM;
-    if ((m + kRankWaves - 1) / kRankWaves >= (1ll << 31)) return PA_E_RANGE;
+    if (m >= (1ll << 32) / kWave) return PA_E_RANGE;   // work-items of the launch
     if (m == 0) return PA_OK;
     if (!dist || !rows || !cand) return PA_E_NULL;
     const unsigned lds = (unsigned)(kRankWaves * d * sizeof(float));
@@ -716,7 +720,6 @@ extern "C" int pa_graph_prune_rows(int32_t *selected, const void *rows_hi_f16,
                                    float scale2, void *stream_) {
     if (n < 0 || k < 1 || k > 256 || m_keep < 1) return PA_E_SHAPE;
     if (d <= 0 || d % kChunk) return PA_E_DIM;
-    if (n >= (1ll << 31)) return PA_E_RANGE;
     if (n == 0) return PA_OK;
     if (!selected || !rows_hi_f16 || !rows_lo_f16 || !norm || !cand || !cand_dist)
         return PA_E_NULL;
@@ -725,15 +728,21 @@ extern "C" int pa_graph_prune_rows(int32_t *selected, const void *rows_hi_f16,
     a.lo = reinterpret_cast<const _Float16 *>(rows_lo_f16);
     a.norm = norm, a.cand = cand, a.cand_dist = cand_dist, a.selected = selected;
     a.n = n, a.d = d, a.k = k, a.m_keep = m_keep, a.fill = fill, a.scale2 = scale2;
-    prune_rows_kernel<<<(unsigned)n, 512, 0, (hipStream_t)stream_>>>(a);
-    return (int)hipGetLastError();
+    // a launch holds fewer than 2^32 work-items: at most 2^22 nodes of 512
+    for (a.first = 0; a.first < n; a.first += kLaunchNodes) {
+        const int64_t count = n - a.first < kLaunchNodes ? n - a.first : kLaunchNodes;
+        prune_rows_kernel<<<(unsigned)count, 512, 0, (hipStream_t)stream_>>>(a);
+        const hipError_t err = hipGetLastError();
+        if (err != hipSuccess) return (int)err;
+    }
+    return PA_OK;
 }
 
 extern "C" int pa_graph_prune(int32_t *selected, const float *pair,
                               const float *cand_dist, int64_t n, int k,
                               int m_keep, int fill, void *stream_) {
     if (n < 0 || k < 1 || k > 512 || m_keep < 1) return PA_E_SHAPE;
-    if ((n + 3) / 4 >= (1ll << 31)) return PA_E_RANGE;
+    if (n >= (1ll << 32) / kWave) return PA_E_RANGE;   // work-items of the launch
     if (n == 0) return PA_OK;
     if (!selected || !pair || !cand_dist) return PA_E_NULL;
     prune_kernel<<<(unsigned)((n + 3) / 4), 256, 0, (hipStream_t)stream_>>>(

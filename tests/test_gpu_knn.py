@@ -251,3 +251,23 @@ def test_pruning_straight_from_the_rows(n, d, k, m_keep, fill, device):
     with pytest.raises(RuntimeError):
         kernels.graph_prune_rows(x, cand[:, :1].expand(-1, 300).contiguous(),
                                  cand_d[:, :1].expand(-1, 300).contiguous(), m_keep, fill)
+
+
+def test_pruning_of_more_nodes_than_one_launch_takes(device):
+    """A launch holds fewer than 2^32 work-items, 2^22 nodes of 512: more nodes
+    go in several launches, and the last ones are pruned like the first."""
+    n, k, d = (1 << 22) + 1000, 8, 64
+    print('prune rows, nodes', n, flush=True)
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(2000, d, generator=g).to(device)
+    cand = torch.stack([torch.randperm(2000, generator=g)[:k] for _ in range(1000)]).to(device)
+    cand_d = torch.sort(torch.rand(1000, k, generator=g) * 100 + 60, dim=-1).values.to(device)
+    reps = -(-n // 1000)
+    got = kernels.graph_prune_rows(x, cand.repeat(reps, 1)[:n].contiguous(),
+                                   cand_d.repeat(reps, 1)[:n].contiguous(), 4, True)
+    torch.cuda.synchronize()
+    assert got.shape == (n, 4)
+    assert int(got.min()) >= 0 and int(got.max()) < k
+    # node i has the lists of node i % 1000: every block of 1000 nodes alike
+    assert torch.equal(got[:1000], got[-1000:].roll(n % 1000, 0))
+    assert torch.equal(got[:1000], got[(1 << 22):(1 << 22) + 1000].roll((1 << 22) % 1000, 0))
