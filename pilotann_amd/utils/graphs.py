@@ -215,20 +215,20 @@ def reachable(adj: torch.Tensor, sources: torch.Tensor, reverse: bool = False):
     return mark
 
 
-def _add_edge(adj, protected, u: int, v: int):
-    """Edge u -> v: into the row's first free slot, else over its farthest
-    neighbour that is not itself an edge added here."""
-    row = adj[u]
+def _add_edge(row, protected, u: int, v: int):
+    """Edge u -> v into ``row``, the row of u (a view, changed in place): into
+    its first free slot, else over its farthest neighbour that is not itself
+    an edge added here."""
     if u == v or bool((row == v).any()):
         return
     free = torch.nonzero(row < 0).flatten()
     if free.numel():
-        adj[u, int(free[0])] = v
+        row[int(free[0])] = v
         return
-    deg = adj.size(1)
+    deg = row.numel()
     if int(protected[u]) >= max(1, deg // 4):
         return
-    adj[u, deg - 1 - int(protected[u])] = v
+    row[deg - 1 - int(protected[u])] = v
     protected[u] += 1
 
 
@@ -280,9 +280,14 @@ def connect_graph(x: torch.Tensor, adj: torch.Tensor, hub: int = None,
             d = norms.unsqueeze(0) - 2.0 * (q @ xf[inside].T)
             nearest.append(inside[torch.argmin(d, -1)])
         nearest = torch.cat(nearest)
+        # the rows that get edges, edited on the host and written back
+        touched = torch.unique(torch.cat([cut, nearest]))
+        rows = adj[touched].cpu()
+        place = {node: i for i, node in enumerate(touched.tolist())}
         for u, t in zip(cut.tolist(), nearest.tolist()):
-            _add_edge(adj, protected, t, u)
-            _add_edge(adj, protected, u, t)
+            _add_edge(rows[place[t]], protected, t, u)
+            _add_edge(rows[place[u]], protected, u, t)
+        adj[touched] = rows.to(dev)
     fwd = reachable(adj, hub_t)
     bwd = reachable(adj, hub_t, reverse=True)
     return max_rounds if bool((fwd & bwd).all()) else -1
