@@ -438,6 +438,8 @@ def graph_prune_rows(rows: torch.Tensor, cand: torch.Tensor, cand_dist: torch.Te
     _require(cand.device == rows.device == cand_dist.device, 'one device')
     n, k = cand.shape
     _require(1 <= k <= 256, '1 <= k <= 256')
+    if n == 0:
+        return torch.empty(0, int(m_keep), dtype=torch.long, device=rows.device)
     _require(int(cand.max()) < rows.size(0), 'cand < rows.size(0)')
     parts = HalfRows(rows)
     low = parts.low(rows)
