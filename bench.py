@@ -60,8 +60,8 @@ CONFIGS = {
                entry='router32x32', queries=10_000, k=10,
                ef_sweep=[32, 64, 128], seed=201),
     # the memory-bounded case: 10M x 768, 2.5M reduced rows and their graph
-    # on the device.  By default only the device stage is built, in two
-    # minutes: the subgraph on a seeded random quarter of the nodes and no
+    # on the device.  By default only the device stage is built, in under a
+    # minute: the subgraph on a seeded random quarter of the nodes and no
     # full graph, hence no refine and no end-to-end recall (the recall
     # reported is that of the candidate lists); --full-index builds the whole
     # index (four minutes) and measures the whole search.
