@@ -171,6 +171,7 @@ def build_index(cfg, device, stage_cache=None):
     del x
     torch.cuda.empty_cache()
     index.to(device)
+    cfg['index_build_seconds'] = round(time.time() - t0, 1)
     log(f'[bench] index built {time.time() - t0:.1f}s, '
         f'sampled {index.nodelist.numel()} of {cfg["n"]}')
     if stage_cache:
@@ -664,6 +665,8 @@ def main():
                           'graph, no refine)' if index.fullgraph is None else
                           'whole search: device candidates, then host refine'),
             'stage': 'routing_cuda + traverse_cuda (GPU search stage)',
+            # data, ground truth and the index on the device, when built here
+            'index_build_seconds': cfg.get('index_build_seconds'),
         },
         'roofline': stage_record(t, B, key),
     }
