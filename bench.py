@@ -751,6 +751,37 @@ def context_figures(line, args, cfg, index, stage, query, target, ef,
         'same_results': bool(torch.equal(big_D[-B:], out_D))}
     del big_q, big_EI, big_ED, big_I, big_D
 
+    # context: the same steps with two batches in flight, as a serving loop
+    # keeps them: steps alternate between two streams (each with its own
+    # outputs; the library keeps scratch memory per stream), so the searches of
+    # one step fill the wavefront slots that the last searches of the step
+    # before leave empty
+    streams = [torch.cuda.Stream(device=device) for _ in range(2)]
+    outs = [(torch.empty(B, 4, ef, dtype=torch.long, device=device),
+             torch.empty(B, 4, ef, dtype=torch.float, device=device)) for _ in range(2)]
+
+    def alternate(count):
+        for i in range(count):
+            with torch.cuda.stream(streams[i % 2]):
+                EP_I, EP_D = stage.entries()
+                stage.kernels.traverse_prepared(
+                    outs[i % 2][0], outs[i % 2][1], stage.graph, index.storage_cuda,
+                    stage.query_cuda, EP_I, EP_D, None)
+    torch.cuda.synchronize()
+    alternate(4)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    alternate(args.steps)
+    torch.cuda.synchronize()
+    t_two = time.perf_counter() - t0
+    line['config']['two_batches_in_flight'] = {
+        'what': 'the timed steps alternating between two streams',
+        'steps': args.steps, 'ms_per_step': round(1e3 * t_two / args.steps, 4),
+        'queries_per_s': round(args.steps * B / t_two, 1),
+        'same_results': bool(torch.equal(outs[0][1], out_D) and
+                             torch.equal(outs[1][1], out_D))}
+    del outs
+
     if index.fullgraph is not None:
         chunk = 1000 if B % 1000 == 0 else B
         index.search(query, k=k, ef_search=ef, chunk_size=chunk)
