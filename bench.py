@@ -751,12 +751,34 @@ def context_figures(line, args, cfg, index, stage, query, target, ef,
         'same_results': bool(torch.equal(big_D[-B:], out_D))}
     del big_q, big_EI, big_ED, big_I, big_D
 
+
+    if index.fullgraph is not None:
+        chunk = 1000 if B % 1000 == 0 else B
+        index.search(query, k=k, ef_search=ef, chunk_size=chunk)
+        t0 = time.perf_counter()
+        top_I, top_D = index.search(query, k=k, ef_search=ef, chunk_size=chunk)
+        t_e2e = time.perf_counter() - t0
+        from pilotann_amd import utils as _utils
+        line['config']['end_to_end'] = {
+            'api': 'IndexStaged.search', 'chunk_size': chunk,
+            'queries_per_s': round(B / t_e2e, 1),
+            'recall_at_k': round(_utils.recall(top_I, target), 4)}
+        line['config']['end_to_end_device_refine'] = device_refine_figures(
+            cfg, index, stage, query, target, ef, (top_I, top_D))
+        line['end_to_end_qps_host_refine'] = \
+            line['config']['end_to_end']['queries_per_s']
+        line['end_to_end_qps_device_refine'] = \
+            line['config']['end_to_end_device_refine']['queries_per_s']
+
     # context: the same steps with two batches in flight, as a serving loop
     # keeps them: steps alternate between two streams (each with its own
     # outputs; the library keeps scratch memory per stream), so the searches of
     # one step fill the wavefront slots that the last searches of the step
     # before leave empty
-    streams = [torch.cuda.Stream(device=device) for _ in range(2)]
+    # (the index's own pair of streams where it has one: streams made later
+    # can share a hardware queue, and work on one queue does not overlap)
+    streams = getattr(index, '_streams', None) or \
+        [torch.cuda.Stream(device=device) for _ in range(2)]
     outs = [(torch.empty(B, 4, ef, dtype=torch.long, device=device),
              torch.empty(B, 4, ef, dtype=torch.float, device=device)) for _ in range(2)]
 
@@ -778,27 +800,13 @@ def context_figures(line, args, cfg, index, stage, query, target, ef,
         'what': 'the timed steps alternating between two streams',
         'steps': args.steps, 'ms_per_step': round(1e3 * t_two / args.steps, 4),
         'queries_per_s': round(args.steps * B / t_two, 1),
+        # algorithmic bytes of all steps over the whole time (launches
+        # overlap: not a per-launch figure like roofline.achieved)
+        'aggregate_GBps': round(args.steps * launch_bytes / t_two / 1e9, 1),
+        'aggregate_frac': round(args.steps * launch_bytes / t_two / 1e9 / HBM_PEAK_GBS, 4),
         'same_results': bool(torch.equal(outs[0][1], out_D) and
                              torch.equal(outs[1][1], out_D))}
     del outs
-
-    if index.fullgraph is not None:
-        chunk = 1000 if B % 1000 == 0 else B
-        index.search(query, k=k, ef_search=ef, chunk_size=chunk)
-        t0 = time.perf_counter()
-        top_I, top_D = index.search(query, k=k, ef_search=ef, chunk_size=chunk)
-        t_e2e = time.perf_counter() - t0
-        from pilotann_amd import utils as _utils
-        line['config']['end_to_end'] = {
-            'api': 'IndexStaged.search', 'chunk_size': chunk,
-            'queries_per_s': round(B / t_e2e, 1),
-            'recall_at_k': round(_utils.recall(top_I, target), 4)}
-        line['config']['end_to_end_device_refine'] = device_refine_figures(
-            cfg, index, stage, query, target, ef, (top_I, top_D))
-        line['end_to_end_qps_host_refine'] = \
-            line['config']['end_to_end']['queries_per_s']
-        line['end_to_end_qps_device_refine'] = \
-            line['config']['end_to_end_device_refine']['queries_per_s']
 
     if args.config == 'c3' and cfg['decay'] == 0 and not args.n_base:
         line['config']['power_law_spectrum'] = spectrum_twin(cfg, device, args)
