@@ -198,7 +198,8 @@ def train_stage_only(index, x, cfg):
     print('build', index.graph_type, 'on', nodelist.numel(), 'sampled nodes')
     sub = xr[nodelist.to(xr.device)]
     sg_indptr, sg_indices = utils.graph_init(
-        sub, index.graph_type, index.n_neighbors, compute_dtype=torch.float16)
+        sub, index.graph_type, index.n_neighbors, compute_dtype=torch.float16,
+        seed=index.seed + 1)
     del sub
     glob_ids = torch.where(sg_indices >= 0, nodelist[sg_indices.clamp(min=0)],
                            torch.full_like(sg_indices, -1))

@@ -172,7 +172,7 @@ class IndexStaged(nn.Module):
         print('build', self.graph_type)
         graph = utils.graph_init(xr, graph_type=self.graph_type,
                                  n_neighbors=self.n_neighbors,
-                                 compute_dtype=half)
+                                 compute_dtype=half, seed=self.seed)
         self.register_module('fullgraph', GraphModule(graph[0], graph[1]))
 
         print('sampling', self.sample_ratio)

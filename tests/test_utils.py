@@ -158,10 +158,13 @@ def test_connectivity_pass_joins_separated_clusters():
     n, d, deg = 4000, 32, 16
     x = utils.gaussian_mixture(n, d, 16, 0.05, seed=8)
     for graph_type in ['nsw', 'nsg']:
-        _, loose = utils.graph_init(x, graph_type, deg, connect=False)
+        # every pool from the whole set: the table the pass is there for
+        _, loose = utils.graph_init(x, graph_type, deg, connect=False,
+                                    insertion_order=False)
         loose = loose.view(n, deg)
         assert not bool(utils.reachable(loose, torch.tensor([0])).all())
-        indptr, indices = utils.graph_init(x, graph_type, deg)
+        indptr, indices = utils.graph_init(x, graph_type, deg,
+                                           insertion_order=False)
         rows = indices.view(n, deg)
         for start in (0, 1234, n - 1):
             assert bool(utils.reachable(rows, torch.tensor([start])).all())
@@ -186,3 +189,42 @@ def test_connectivity_pass_joins_separated_clusters():
         # (0.08 on the table without the pass: one cluster of sixteen; the
         # bridges are few, so a greedy search does not always find them)
         assert utils.recall(torch.from_numpy(out_I), target) > 0.5
+
+
+def test_insertion_order_makes_the_graph_navigable_across_clusters():
+    """Pools taken in insertion order (a node's nearest among the nodes
+    before it in a seeded random order): the early nodes' long edges join the
+    clusters without the connectivity pass, and a search from one fixed entry
+    finds the neighbours of queries of every cluster far better than on the
+    table of nearest neighbours in the whole set with its few bridges."""
+    import numpy as np
+    import oracle
+    n, d, deg = 4000, 32, 16
+    x = utils.gaussian_mixture(n, d, 16, 0.05, seed=8)
+    q = utils.gaussian_mixture(64, d, 16, 0.05, seed=9, center_seed=8)
+    target = utils.brute_force_topk(q, x, 10)
+    init_I = torch.zeros(64, 1, dtype=torch.long)
+    init_D = (q - x[0]).square().sum(-1, keepdim=True)
+    score = {}
+    for ordered in (False, True):
+        indptr, indices = utils.graph_init(x, 'nsw', deg, connect=not ordered,
+                                           insertion_order=ordered, seed=3)
+        rows = indices.view(n, deg)
+        for start in (0, 1234, n - 1):
+            assert bool(utils.reachable(rows, torch.tensor([start])).all())
+            assert bool(utils.reachable(rows, torch.tensor([start]), reverse=True).all())
+        valid = rows >= 0
+        assert (valid[:, :-1] | ~valid[:, 1:]).all()
+        assert not (rows == torch.arange(n).unsqueeze(1)).any()
+        srt = torch.sort(torch.where(valid, rows, -torch.arange(1, deg + 1)), 1).values
+        assert (srt[:, 1:] != srt[:, :-1]).all()
+        out_I = np.empty((64, 10), np.int64)
+        out_D = np.empty((64, 10), np.float32)
+        oracle.traverse_cpu(out_I, out_D, init_I.numpy(), init_D.numpy().copy(),
+                            indptr.numpy(), indices.numpy(), x.numpy(), q.numpy(), 64)
+        score[ordered] = utils.recall(torch.from_numpy(out_I), target)
+    print('recall@10 from one entry, whole-set pools / insertion order:', score)
+    assert score[True] > 0.9 and score[True] > score[False]
+    # same seed, same graph
+    again = utils.graph_init(x, 'nsw', deg, connect=False, seed=3)[1]
+    assert torch.equal(again, indices)
