@@ -358,12 +358,16 @@ struct OpenList {
         bool bottom; // it is on level kDepth
     };
     __device__ __forceinline__ Leaf walk_to_large_leaf() const {
-        const Choice ch = choices<true>();
-        int j = 1;
+        return walk_below(choices<true>(), 0, 1);
+    }
+    // The walk from node j on level DONE down to a leaf (the levels above
+    // were taken elsewhere).
+    __device__ __forceinline__ Leaf walk_below(const Choice &ch, const int DONE,
+                                               int j) const {
         bool bottom = true;  // the walk reached level kDepth
         int walked_key = 0;  // key of node j when its level is an LDS level
 #pragma unroll
-        for (int L = 1; L <= kDepth; ++L) {
+        for (int L = DONE + 1; L <= kDepth; ++L) {
             if (L == kDepth && 2 * j > kSize) {
                 bottom = false;
                 break;
@@ -387,6 +391,47 @@ struct OpenList {
         else
             leaf.key = kind(kDepth - 1) >= 3 ? walked_key : key_of(kind(kDepth - 1), j);
         return leaf;
+    }
+    // The seven register levels of that walk (lists of 256 cells and more,
+    // where they are complete) together with a wavefront maximum of `x`,
+    // which comes back in lane 63: the six v_max_i32_dpp of the maximum each
+    // need two wait states after the one before, and the three scalar
+    // instructions of a level fill them, where apart they would be s_nop.
+    // Returns the node on level 7.
+    static constexpr bool kFusedTop = kDepth >= 8;
+    __device__ __forceinline__ static int top_levels_and_wave_max(const Choice &ch,
+                                                                  int &x) {
+        int j, t;
+        asm("s_bitcmp1_b64 %[a], 3\n\t"
+            "s_addc_u32 %[j], 2, 0\n\t"
+            "v_max_i32_dpp %[x], %[x], %[x] quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf\n\t"
+            "s_lshl1_add_u32 %[j], %[j], 1\n\t"
+            "s_bitcmp1_b64 %[a], %[j]\n\t"
+            "s_addc_u32 %[j], %[j], -1\n\t"
+            "v_max_i32_dpp %[x], %[x], %[x] quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf\n\t"
+            "s_lshl1_add_u32 %[j], %[j], 1\n\t"
+            "s_bitcmp1_b64 %[a], %[j]\n\t"
+            "s_addc_u32 %[j], %[j], -1\n\t"
+            "v_max_i32_dpp %[x], %[x], %[x] row_half_mirror row_mask:0xf bank_mask:0xf\n\t"
+            "s_lshl1_add_u32 %[j], %[j], 1\n\t"
+            "s_bitcmp1_b64 %[a], %[j]\n\t"
+            "s_addc_u32 %[j], %[j], -1\n\t"
+            "v_max_i32_dpp %[x], %[x], %[x] row_mirror row_mask:0xf bank_mask:0xf\n\t"
+            "s_lshl1_add_u32 %[j], %[j], 1\n\t"
+            "s_bitcmp1_b64 %[a], %[j]\n\t"
+            "s_addc_u32 %[j], %[j], -1\n\t"
+            "v_max_i32_dpp %[x], %[x], %[x] row_bcast:15 row_mask:0xa bank_mask:0xf\n\t"
+            "s_lshl1_add_u32 %[j], %[j], 1\n\t"
+            "s_bitcmp1_b64 %[b], %[j]\n\t"
+            "s_addc_u32 %[j], %[j], -1\n\t"
+            "v_max_i32_dpp %[x], %[x], %[x] row_bcast:31 row_mask:0xc bank_mask:0xf\n\t"
+            "s_lshl_b32 %[t], %[j], 1\n\t"
+            "s_bitcmp1_b64 %[cd], %[j]\n\t"
+            "s_addc_u32 %[j], %[t], 0"
+            : [j] "=&s"(j), [x] "+v"(x), [t] "=&s"(t)
+            : [a] "s"(ch.a), [b] "s"(ch.b), [cd] "s"(ch.cd)
+            : "scc");
+        return j;
     }
     // SPARSE: the heap is nearly empty (the entries of a query are pushed),
     // so most ancestors of the leaf are (inf, -1), and so is everything below
@@ -511,6 +556,110 @@ struct Results {
         begin_insert(k, v, lane, key);
         finish_insert(lane, key);
     }
+};
+
+// ---- result list of the traversal: sorted keys per lane, entries in a log -------
+//
+// The same set as Results<S> above, kept so that an insert touches no cell by
+// position.  Lane l owns S keys, largest first; the set's maximum is the
+// largest first key, `holder` a lane that has it.  A candidate below the
+// maximum replaces it: in the holder lane the first key leaves and the new
+// key is sorted in, one v_med3_i32 per key (new[s] = the new key clamped
+// between old[s + 1] and old[s]); every other lane runs the same
+// instructions with the largest integer for a key, which changes nothing.
+// Then a wavefront maximum over the first keys.  No key is ever looked up by
+// cell, so nothing depends on S but the S clamps: 22 instructions at S = 2,
+// 28 at S = 8, against 33 and 71 for the flat cells of Results<S>.
+// Which node a key belongs to is not kept here: every admitted candidate is
+// also appended to a log in the wavefront's device memory (ResultLog), and
+// the final set is read back from the log by its keys.
+template <int S>
+struct ResultKeys {
+    static constexpr int kInf = 0x7f800000;          // float_to_key(+inf)
+    static constexpr int kNegInf = (int)0x807fffff;  // float_to_key(-inf)
+    int key[S];   // this lane's keys, key[0] >= key[1] >= ...
+    int worst;    // uniform: the largest key of the set
+    int holder;   // uniform: a lane whose key[0] is `worst`
+
+    // Empty cells hold +inf (the maximum is +inf until H candidates came),
+    // cells beyond H hold -inf and never win.
+    __device__ __forceinline__ void init(int H, int lane) {
+#pragma unroll
+        for (int s = 0; s < S; ++s) key[s] = lane * S + s < H ? kInf : kNegInf;
+        worst = kInf;
+        holder = 0;
+    }
+    __device__ __forceinline__ static int med3(int a, int b, int c) {
+        int r;
+        asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+        return r;
+    }
+    // Caller has checked k < worst.  In two parts for a caller that computes
+    // the wavefront maximum of the first keys itself (`reduced`: any register
+    // whose lane 63 holds it).
+    __device__ __forceinline__ int replace_worst(int k, int lane) {
+        const int kk = lane == holder ? k : 0x7fffffff;
+#pragma unroll
+        for (int s = 0; s + 1 < S; ++s) key[s] = med3(key[s + 1], key[s], kk);
+        key[S - 1] = min(key[S - 1], kk);
+        return key[0];
+    }
+    __device__ __forceinline__ void set_worst(int reduced) {
+        worst = __builtin_amdgcn_readlane(reduced, kWave - 1);
+        holder = __builtin_ctzll(__ballot(key[0] == worst));
+    }
+    __device__ __forceinline__ void insert(int k, int lane) {
+        replace_worst(k, lane);
+        worst = wave_max_key(key[0]);
+        holder = __builtin_ctzll(__ballot(key[0] == worst));
+    }
+};
+
+// The log behind ResultKeys: (key, value) of every admitted candidate, in the
+// wavefront's device memory.  An entry whose key is below the set's maximum
+// is in the set (an entry leaves the set as its maximum, and the maximum only
+// falls); entries at the maximum are in it or tie with one that is, at most H
+// of them at any time.  So cutting the log down to the entries at or below
+// the maximum leaves fewer than 2H, and a log of 2H + 128 entries always has
+// room for the 64 candidates of a step after a cut.
+struct ResultLog {
+    int2 *entry;   // device memory, capacity entries, 8-byte aligned
+    int n;         // uniform: entries in use
+    int capacity;  // uniform
+
+    __host__ __device__ static constexpr int capacity_for(int H) { return 2 * H + 128; }
+
+    // Lanes whose bit is set in `who` append (k, v), in lane order.
+    __device__ __forceinline__ void append(unsigned long long who, int k, int v,
+                                           int lane) {
+        if ((who >> lane) & 1) entry[n + lane_rank(who)] = make_int2(k, v);
+        n += __popcll(who);
+    }
+    // The wavefront's own stores must be visible to the loads of its other
+    // lanes: both go through the compute unit's cache, program order and a
+    // wait for the stores are enough.
+    __device__ __forceinline__ static void settle() {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");
+    }
+    // Drops the entries above `worst`, in place, order kept.
+    __device__ __forceinline__ void cut(int worst, int lane) {
+        settle();
+        int m = 0;
+        for (int base = 0; base < n; base += kWave) {
+            const int i = base + lane;
+            int2 e = make_int2(0x7fffffff, -1);
+            if (i < n) e = entry[i];
+            const bool keep = i < n && e.x <= worst;
+            const unsigned long long mask = __ballot(keep);
+            // m + rank <= i: the write lands on an entry already read
+            if (keep) entry[m + lane_rank(mask)] = e;
+            m += __popcll(mask);
+        }
+        n = m;
+        settle();
+    }
+    __device__ __forceinline__ bool nearly_full() const { return n > capacity - kWave; }
 };
 
 // ---- visited set ----------------------------------------------------------------

@@ -128,8 +128,6 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
         float cand_key[kWave];
         float query[DP8 ? query_floats(8 * DP8) : 4];
         int2 heap[kHeapCells];  // open list tail; the final sort reuses it
-        int res_key[Results<S>::kLdsKeys];  // result list: keys, unless in registers
-                                            // (values: the slot's memory)
     };
     __shared__ __align__(16) Lds lds;
     extern __shared__ __align__(16) float query_any_length[];  // DP8 == 0 only
@@ -146,8 +144,12 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
     const bool use_cache = a.n_storage <= (0xffff << kSeenCacheLog2);
     const int deg = a.deg;
     uint32_t *seen = a.seen + (size_t)blockIdx.x * (size_t)a.slot_stride;
-    // after the visited slice and the result values (H of them, rounded up)
-    open.deep = reinterpret_cast<int2 *>(seen + a.words_per_slot + (H + kWave - 1) / kWave * kWave);
+    // after the visited slice: the log of admitted candidates, then the
+    // levels of the open list kept in device memory
+    ResultLog log;
+    log.entry = reinterpret_cast<int2 *>(seen + a.words_per_slot);
+    log.capacity = ResultLog::capacity_for(H);
+    open.deep = log.entry + ResultLog::capacity_for(H);
 
     for (;;) {
         int q = 0;
@@ -172,10 +174,9 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
             qv[query_slot(i, dp >> 3)] = a.query[(size_t)q * dp + i];
         for (int i = lane; i < kSeenCache; i += kWave) seen_cache[i] = 0xffffffffu;
         open.reset(lane);
-        Results<S> res;
-        res.rk = lds.res_key;
-        res.rv = reinterpret_cast<int *>(seen + a.words_per_slot);
+        ResultKeys<S> res;
         res.init(H, lane);
+        log.n = 0;
         // The clearing stores must have reached the cache level where the
         // atomic ORs are performed before the first OR is issued.  Only this
         // wavefront touches the slice, so waiting for its own stores is
@@ -220,14 +221,11 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
         // return is the root of the open list as it stands after the last
         // insert, so once a step's inserts are done the next step's node is
         // certain: its neighbours' visited bits are tested and set *before*
-        // the pop (the atomics are in flight while the pop sifts).  Its row of
-        // neighbour ids is needed for that, and is requested even earlier,
-        // before the inserts, for the node that will most likely be the root
-        // after them: the best new candidate if it beats the present root and
-        // the admission bound, else the present root.  That load is only a
-        // read; when the guess is wrong the row is loaded again.  If the
+        // the pop (the atomics are in flight while the pop sifts).  If the
         // search ends at the next pop instead, the marks set for a node that
         // is never expanded are harmless: the slice is cleared per query.
+        // (Requesting that node's row of neighbour ids even earlier, before
+        // the inserts, for the most likely next root, measured the same.)
         auto load_row = [&](int r) -> int {
             int row = -1;
             if (r >= 0 && lane < deg) row = a.adj[(size_t)r * deg + lane];
@@ -262,7 +260,6 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
             PA_TIMER(0);
             if (u == -1 || uk >= res.worst) break;
             n_expand += 1;
-            int guess = -3, guess_row = -1;
             bool popped = false;  // the pop has been finished
             if (u >= 0) {
                 n_adj += deg;
@@ -284,49 +281,48 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
 
                     const int d = float_to_key(lane < n ? cand_key[lane] : INFINITY);
                     const int id = lane < n ? cand_id[lane] : -1;
-                    // most likely next node; first candidate on ties, as the
-                    // rise of an equal key stops below the older one
-                    const int d_min = -wave_max_key(-d);
-                    guess = Open::rl(open.Av, 1);
-                    if (d_min < Open::rl(open.Ak, 1) && d_min < res.worst)
-                        guess = __builtin_amdgcn_readlane(
-                            id, __builtin_ctzll(__ballot(d == d_min)));
-                    guess_row = load_row(guess);
-
                     // heap_update, traverse_cpu.cpp:25-39, in adjacency order
                     unsigned long long todo = __ballot(d < res.worst);
+                    unsigned long long admitted = 0;
                     while (todo) {
                         const int j = __builtin_ctzll(todo);
                         todo &= todo - 1;
                         const int dj = __builtin_amdgcn_readlane(d, j);
                         if (dj >= res.worst) continue;
                         const int vj = __builtin_amdgcn_readlane(id, j);
-                        int mine[S];
-                        res.begin_insert(dj, vj, lane, mine);
-                        const typename Open::Leaf leaf = open.walk_to_large_leaf();
-                        res.finish_insert(lane, mine);
+                        typename Open::Leaf leaf;
+                        if (Open::kFusedTop) {
+                            // the result list's new maximum and the top of
+                            // the open list's walk in one instruction stream
+                            const typename Open::Choice ch = open.template choices<true>();
+                            int first = res.replace_worst(dj, lane);
+                            const int j7 = Open::top_levels_and_wave_max(ch, first);
+                            res.set_worst(first);
+                            leaf = open.walk_below(ch, 7, j7);
+                        } else {
+                            leaf = open.walk_to_large_leaf();
+                            res.insert(dj, lane);
+                        }
                         open.replace_leaf(leaf, dj, vj, lane);
-                        n_admit += 1;
+                        admitted |= 1ull << j;
+                    }
+                    if (admitted) {
+                        n_admit += __popcll(admitted);
+                        log.append(admitted, d, id, lane);
+                        if (log.nearly_full()) log.cut(res.worst, lane);
                     }
                     PA_TIMER(4);
                 }
             }
             if (!popped) open.pop_finish(lane);
-            const int r = Open::rl(open.Av, 1);
-            v = r == guess ? guess_row : load_row(r);
+            v = load_row(Open::rl(open.Av, 1));
             before = test_and_set(v);
             PA_TIMER(1);
         }
 
-        // traverse_cpu.cpp:138-148: storage rows -> global ids, then the
-        // entries compete for a result slot.
-        wave_sync();
-#pragma unroll
-        for (int s = 0; s < S; ++s) {
-            const int row = res.rv[lane * S + s];
-            if (row >= 0) res.rv[lane * S + s] = a.gid[row];
-        }
-        wave_sync();
+        // traverse_cpu.cpp:138-148: the entries compete for a result slot.  A
+        // log value below -1 is the global id -2 - value of an entry, the
+        // others are storage rows.
         for (int base = 0; base < a.n_init; base += kWave) {
             const int i = base + lane;
             int u = -1;
@@ -338,25 +334,53 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
             }
             const int dk = float_to_key(d);
             unsigned long long todo = __ballot(u >= 0 && dk < res.worst);
+            unsigned long long admitted = 0;
             while (todo) {
                 const int j = __builtin_ctzll(todo);
                 todo &= todo - 1;
                 const int dj = __builtin_amdgcn_readlane(dk, j);
                 if (dj >= res.worst) continue;
-                res.insert(dj, __builtin_amdgcn_readlane(u, j), lane);
+                res.insert(dj, lane);
+                admitted |= 1ull << j;
+            }
+            if (admitted) {
+                log.append(admitted, dk, -2 - u, lane);
+                if (log.nearly_full()) log.cut(res.worst, lane);
             }
         }
 
-        // traverse_cpu.cpp:150-162: best first.  Sort the H cells (padded to
-        // a power of two with +inf) in the LDS the open list no longer needs.
+        // traverse_cpu.cpp:150-162: best first.  The set is read back from
+        // the log — every entry below the maximum, and of those at the
+        // maximum as many as make H — into the LDS the open list no longer
+        // needs, padded to a power of two with +inf, and sorted there.
         wave_sync();
         for (int i = lane; i < a.sort_n; i += kWave)
             okey[i] = INFINITY, oval[i] = -1;
-        wave_sync();
-#pragma unroll
-        for (int s = 0; s < S; ++s) {
-            const int e = lane * S + s;
-            if (e < H) okey[e] = key_to_float(res.cell_key(lane, s)), oval[e] = res.rv[e];
+        ResultLog::settle();
+        int n_below = 0;
+        for (int base = 0; base < log.n; base += kWave) {
+            const int i = base + lane;
+            n_below += __popcll(__ballot(i < log.n && log.entry[i].x < res.worst));
+        }
+        {
+            int at_below = 0, at_worst = n_below;
+            for (int base = 0; base < log.n; base += kWave) {
+                const int i = base + lane;
+                int2 e = make_int2(0x7fffffff, -1);
+                if (i < log.n) e = log.entry[i];
+                const bool below = i < log.n && e.x < res.worst;
+                const bool tie = i < log.n && e.x == res.worst;
+                const unsigned long long mb = __ballot(below), mt = __ballot(tie);
+                int place = -1;
+                if (below) place = at_below + lane_rank(mb);
+                if (tie) place = at_worst + lane_rank(mt);
+                if (place >= 0 && place < H) {
+                    okey[place] = key_to_float(e.x);
+                    oval[place] = e.y < -1 ? -2 - e.y : a.gid[e.y];
+                }
+                at_below += __popcll(mb);
+                at_worst += __popcll(mt);
+            }
         }
         wave_sync();
         for (int size = 2; size <= a.sort_n; size <<= 1) {
@@ -599,9 +623,9 @@ int make_plan(int64_t n_storage, int64_t batch, int dp, int ef_total, Plan *p) {
     if (slots < 1) slots = 1;
     p->n_slots = (int)slots;
     p->words_per_slot = round_up((n_storage + 31) / 32, kSlotAlignWords);
-    // a slot: the visited slice, the values of the result list, the levels
-    // of the open list that are kept in device memory (8 bytes a cell)
-    p->slot_stride = p->words_per_slot + round_up(p->H, kWave) +
+    // a slot: the visited slice, the log of admitted candidates, the levels
+    // of the open list that are kept in device memory (8 bytes an entry or cell)
+    p->slot_stride = p->words_per_slot + 2 * ResultLog::capacity_for(p->H) +
                      round_up(2 * open_list_deep_cells(p->H, deep_from(p->H)), kWave);
     p->workspace_bytes =
         kWorkCounterBytes + (size_t)p->n_slots * p->slot_stride * 4;
