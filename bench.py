@@ -16,7 +16,8 @@ and on the device, are the top-level fields `end_to_end_qps_host_refine` and
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--config c1..c5]
                     [--n-base N] [--queries B] [--ef EF] [--decay X] [--curve]
-                    [--no-cpu-baseline] [--no-context] [--copy-calibration]
+                    [--no-cpu-baseline] [--no-context] [--power-law-twin]
+                    [--copy-calibration]
 """
 import argparse
 import contextlib
@@ -558,6 +559,11 @@ def main():
                     help="only time the graph builder's nearest-neighbour "
                          "kernel (pa_knn) on the configuration's base set "
                          "against itself, print its rate and exit")
+    ap.add_argument('--power-law-twin', action='store_true',
+                    help='also build the configuration on data with a '
+                         'power-law spectrum (exponent 0.5) and measure recall '
+                         'and rate over a range of ef there (a second index '
+                         'build; context, not part of `value`)')
     ap.add_argument('--copy-calibration', action='store_true',
                     help='only run a plain 1 GiB device copy five times (to '
                          'scale the FETCH_SIZE / WRITE_SIZE counters) and exit')
@@ -711,9 +717,9 @@ def context_figures(line, args, cfg, index, stage, query, target, ef,
                     launch_bytes, out_D):
     """Not part of `value`: the same step with its inputs and outputs
     crossing PCIe (pageable host memory), the launch over a fourfold batch,
-    the whole three-stage search (`IndexStaged.search`: rotation on the
-    host, entries, pipeline), and the headline workload's twin with a
-    power-law spectrum."""
+    the whole three-stage search (`IndexStaged.search`: rotation, entries,
+    pipeline), the same steps with two batches in flight and, on request, the
+    workload's twin with a power-law spectrum."""
     B, k, dp, device = stage.B, cfg['k'], cfg['dp'], stage.device
     host_q = stage.query_rot[:, :dp].contiguous()
     torch.cuda.synchronize()
@@ -809,7 +815,7 @@ def context_figures(line, args, cfg, index, stage, query, target, ef,
                              torch.equal(outs[1][1], out_D))}
     del outs
 
-    if args.config == 'c3' and cfg['decay'] == 0 and not args.n_base:
+    if args.power_law_twin:
         line['config']['power_law_spectrum'] = spectrum_twin(cfg, device, args)
 
 

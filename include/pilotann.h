@@ -294,8 +294,9 @@ int pa_graph_prune(int32_t *selected, const float *pair, const float *cand_dist,
  * made inside the kernel and never stored.  rows_hi_f16 / rows_lo_f16 hold
  * every row as two half-precision parts (row * s = hi + lo, rows of d
  * elements, d % 64 == 0, padded with zeros), norm [rows] the squared lengths
- * of the scaled rows, cand [n * k] the candidates' row numbers (closest first,
- * -1 after the last), cand_dist [n * k] their squared distances to the node in
+ * of the scaled rows, n_rows the number of rows behind them, cand [n * k] the
+ * candidates' row numbers (closest first, -1 after the last; a number at or
+ * beyond n_rows counts as -1 and nothing is read for it), cand_dist [n * k] their squared distances to the node in
  * the rows' own units and scale2 = s * s.  A pair's distance is
  * |a|^2 + |b|^2 - 2 (hi.hi + hi.lo + lo.hi): the float32 value to about 22
  * bits.  selected as for pa_graph_prune.  Device pointers; enqueued on
@@ -304,8 +305,8 @@ int pa_graph_prune(int32_t *selected, const float *pair, const float *cand_dist,
 int pa_graph_prune_rows(int32_t *selected, const void *rows_hi_f16,
                         const void *rows_lo_f16, const float *norm,
                         const int64_t *cand, const float *cand_dist, int64_t n,
-                        int d, int k, int m_keep, int fill, float scale2,
-                        void *stream);
+                        int64_t n_rows, int d, int k, int m_keep, int fill,
+                        float scale2, void *stream);
 
 /*
  * The reference's operator hooks (extension/ops_cpu.cpp:8-95,

@@ -40,8 +40,8 @@ _SIGNATURES = {
     'pa_knn_rerank': (_int, [_vp, _vp, _vp, _i64, _i64, _i64, _int, _int, _vp]),
     'pa_knn': (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _int, _int, _vp]),
     'pa_graph_prune': (_int, [_vp, _vp, _vp, _i64, _int, _int, _int, _vp]),
-    'pa_graph_prune_rows': (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _int,
-                            _int, ctypes.c_float, _vp]),
+    'pa_graph_prune_rows': (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _int, _int,
+                            _int, _int, ctypes.c_float, _vp]),
     'pa_heapq_pop': (_int, [_vp, _vp, _i64]),
     'pa_heapq_pushpop': (_int, [_vp, _vp, _i64, ctypes.c_float, _i64]),
     'pa_heapq_replace': (_int, [_vp, _vp, _i64, ctypes.c_float, _i64]),

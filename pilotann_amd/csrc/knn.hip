@@ -484,6 +484,7 @@ struct PruneRowsArgs {
     const float *cand_dist;   // [n, k] squared distances to the node, unscaled
     int32_t *selected;        // [n, m_keep]
     int64_t n, first;         // this launch takes nodes first .. first + gridDim.x
+    int64_t n_rows;           // rows behind hi / lo / norm: a candidate at or beyond is no candidate
     int d, k, m_keep, fill;
     float scale2;             // (scaled / unscaled) squared
 };
@@ -504,17 +505,22 @@ __global__ __launch_bounds__(512, 2) void prune_rows_kernel(PruneRowsArgs a) {
     const int col = lane & 31, half = lane >> 5;
     const int64_t node = a.first + blockIdx.x;
     const int64_t *ids = a.cand + (size_t)node * a.k;
+    // a candidate: a row number inside the set, else -1 (nothing is read for it)
+    auto cand_at = [&](int i) -> int64_t {
+        const int64_t id = i < a.k ? ids[i] : -1;
+        return id < a.n_rows ? id : -1;
+    };
 
     // the candidates' lengths and distances; what lies behind the list
     // repeats the first candidate and can block nothing
     if (t < kRows) {
-        const int64_t id = t < a.k ? ids[t] : -1;
+        const int64_t id = cand_at(t);
         len2[t] = id >= 0 ? a.norm[id] : 0.f;
         reach[t] = id >= 0 ? a.cand_dist[(size_t)node * a.k + t] * a.scale2 : -INFINITY;
     }
     if (t == 0) valid_count = 0;
     __syncthreads();
-    if (t < a.k && ids[t] >= 0) atomicAdd(&valid_count, 1);
+    if (cand_at(t) >= 0) atomicAdd(&valid_count, 1);
 
     // transfers: wavefront w brings rows 32 w .. 32 w + 31 of both parts, 8
     // rows an instruction, lane l the piece that belongs at place l % 8 of row
@@ -524,8 +530,8 @@ __global__ __launch_bounds__(512, 2) void prune_rows_kernel(PruneRowsArgs a) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         const int row = 32 * wave + 8 * i + bring_row;
-        int64_t id = row < a.k ? ids[row] : -1;
-        if (id < 0) id = ids[0] >= 0 ? ids[0] : 0;
+        int64_t id = cand_at(row);
+        if (id < 0) id = cand_at(0) >= 0 ? cand_at(0) : 0;
         from[i] = ((size_t)id * a.d) * 2 + 16u * ((lane & 7) ^ (((8 * i + bring_row) >> 1) & 7));
     }
     const unsigned bring_to =
@@ -716,9 +722,10 @@ extern "C" int pa_knn_rerank(float *dist, const float *rows, const int64_t *cand
 extern "C" int pa_graph_prune_rows(int32_t *selected, const void *rows_hi_f16,
                                    const void *rows_lo_f16, const float *norm,
                                    const int64_t *cand, const float *cand_dist,
-                                   int64_t n, int d, int k, int m_keep, int fill,
-                                   float scale2, void *stream_) {
-    if (n < 0 || k < 1 || k > 256 || m_keep < 1) return PA_E_SHAPE;
+                                   int64_t n, int64_t n_rows, int d, int k,
+                                   int m_keep, int fill, float scale2,
+                                   void *stream_) {
+    if (n < 0 || n_rows < 1 || k < 1 || k > 256 || m_keep < 1) return PA_E_SHAPE;
     if (d <= 0 || d % kChunk) return PA_E_DIM;
     if (n == 0) return PA_OK;
     if (!selected || !rows_hi_f16 || !rows_lo_f16 || !norm || !cand || !cand_dist)
@@ -727,7 +734,8 @@ extern "C" int pa_graph_prune_rows(int32_t *selected, const void *rows_hi_f16,
     a.hi = reinterpret_cast<const _Float16 *>(rows_hi_f16);
     a.lo = reinterpret_cast<const _Float16 *>(rows_lo_f16);
     a.norm = norm, a.cand = cand, a.cand_dist = cand_dist, a.selected = selected;
-    a.n = n, a.d = d, a.k = k, a.m_keep = m_keep, a.fill = fill, a.scale2 = scale2;
+    a.n = n, a.n_rows = n_rows, a.d = d, a.k = k, a.m_keep = m_keep, a.fill = fill;
+    a.scale2 = scale2;
     // a launch holds fewer than 2^32 work-items: at most 2^22 nodes of 512
     for (a.first = 0; a.first < n; a.first += kLaunchNodes) {
         const int64_t count = n - a.first < kLaunchNodes ? n - a.first : kLaunchNodes;

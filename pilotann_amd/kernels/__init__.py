@@ -302,29 +302,40 @@ def entry_distances(query: torch.Tensor, entry_vectors: torch.Tensor):
 
 class HalfRows:
     """Rows prepared for :func:`knn_candidates`: a half-precision copy, scaled
-    into [-1, 1], padded with zeros to whole tiles of the kernel
+    so that a row is about one unit long (root mean square over the set) and
+    clamped to the half range, padded with zeros to whole tiles of the kernel
     (``pa_knn_tile_rows()`` rows, 64 columns: what it reads without bounds
-    checks), and the squared lengths of the scaled rows."""
+    checks), and the squared lengths of the scaled rows.  (Scaling by the
+    largest coordinate instead would push a set with a few large coordinates
+    — outliers, unnormalised embeddings — into the half subnormals.)"""
+
+    HALF_MAX = 60000.0
 
     def __init__(self, rows: torch.Tensor, scale: float = None):
         _check(rows, 'rows', 2, torch.float32, True)
         n, d = rows.shape
         if scale is None:
-            scale = 1.0 / max(float(rows.abs().max()), 1e-30) if n else 1.0
+            rms = float(rows.square().sum(-1).mean().sqrt()) if n else 1.0
+            scale = 1.0 / max(rms, 1e-30)
         self.n, self.d, self.scale = n, d, scale
         self.tile = int(_lib.lib().pa_knn_tile_rows())
         n_pad, d_pad = -(-max(n, 1) // self.tile) * self.tile, -(-d // 64) * 64
         self.half = torch.zeros(n_pad, d_pad, dtype=torch.float16, device=rows.device)
-        self.half[:n, :d] = rows * scale
         self.norm = torch.zeros(n_pad, dtype=torch.float32, device=rows.device)
-        self.norm[:n] = (rows * scale).square().sum(-1)
+        for lo in range(0, n, 1 << 20):     # in pieces: no second copy of a large set
+            piece = (rows[lo:lo + (1 << 20)] * scale).clamp_(-self.HALF_MAX, self.HALF_MAX)
+            self.half[lo:lo + piece.size(0), :d] = piece
+            self.norm[lo:lo + piece.size(0)] = piece.square().sum(-1)
 
     def low(self, rows: torch.Tensor) -> torch.Tensor:
         """The second half-precision part of ``rows`` (the tensor this set was
         made from): ``rows * scale - half``, same shape and padding as
         ``half``, so that ``half + low`` is the scaled row to about 22 bits."""
         low = torch.zeros_like(self.half)
-        low[:self.n, :self.d] = rows * self.scale - self.half[:self.n, :self.d].float()
+        for lo in range(0, self.n, 1 << 20):
+            hi = min(self.n, lo + (1 << 20))
+            piece = (rows[lo:hi] * self.scale).clamp_(-self.HALF_MAX, self.HALF_MAX)
+            low[lo:hi, :self.d] = piece - self.half[lo:hi, :self.d].float()
         return low
 
     def rows(self, lo: int, hi: int) -> 'HalfRows':
@@ -428,7 +439,8 @@ def graph_prune_rows(rows: torch.Tensor, cand: torch.Tensor, cand_dist: torch.Te
                      m_keep: int, fill: bool):
     """:func:`graph_prune` without the table of pairwise distances
     (``pa_graph_prune_rows``): ``rows`` ``[N, d]`` float32, ``cand`` ``[n, k]``
-    int64 row numbers (closest first, ``-1`` after the last, ``k <= 256``),
+    int64 row numbers (closest first, ``-1`` after the last, ``k <= 256``; a
+    number beyond the rows counts as ``-1``),
     ``cand_dist`` ``[n, k]`` their squared distances to the node.  Returns the
     positions ``[n, m_keep]`` as :func:`graph_prune` does."""
     _check(rows, 'rows', 2, torch.float32, True)
@@ -440,14 +452,14 @@ def graph_prune_rows(rows: torch.Tensor, cand: torch.Tensor, cand_dist: torch.Te
     _require(1 <= k <= 256, '1 <= k <= 256')
     if n == 0:
         return torch.empty(0, int(m_keep), dtype=torch.long, device=rows.device)
-    _require(int(cand.max()) < rows.size(0), 'cand < rows.size(0)')
     parts = HalfRows(rows)
     low = parts.low(rows)
     selected = torch.empty(n, int(m_keep), dtype=torch.int32, device=rows.device)
     with torch.cuda.device(rows.device):
         _lib.check(_lib.lib().pa_graph_prune_rows(
             _ptr(selected), _ptr(parts.half), _ptr(low), _ptr(parts.norm), _ptr(cand),
-            _ptr(cand_dist), n, parts.half.size(1), k, int(m_keep), int(bool(fill)),
+            _ptr(cand_dist), n, rows.size(0), parts.half.size(1), k, int(m_keep),
+            int(bool(fill)),
             float(parts.scale) ** 2, _stream()), 'pa_graph_prune_rows')
     return selected.long()
 

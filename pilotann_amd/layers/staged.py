@@ -142,7 +142,8 @@ class IndexStaged(nn.Module):
         all rows in full dimension, the full graph (prepared once) and the
         rotation."""
         device = self.cuda_device
-        assert device is not None, 'call .to(device) first'
+        assert device is not None and self.storage_cuda is not None, \
+            'call .to(device) first (again after a new build)'
         # not through the cache of prepare_rows: the plain device copy is
         # dropped once its device layout exists
         self.storage_full_cuda = kernels.PreparedRows(
@@ -156,11 +157,20 @@ class IndexStaged(nn.Module):
             self.fullgraph_cuda.indptr, self.fullgraph_cuda.indices)
         return self
 
+    def _drop_device_copies(self):
+        """What :meth:`to` and :meth:`stage_refine` put on the device belongs
+        to the buffers they were made from: after the buffers change (a new
+        build, buffers registered again) the copies are made anew."""
+        self.storage_cuda = self.subgraph_cuda = self.mapping_cuda = None
+        self.fullgraph_cuda = self.storage_full_cuda = self.VT_cuda = None
+        self._full_prepared = None
+
     # -- build: layers/staged.py:141-189 --------------------------------------
     def train(self, x: torch.Tensor):
         assert x.dim() == 2
         assert x.size(-1) == self.d_model
         assert 0.0 < self.sample_ratio <= 1.0
+        self._drop_device_copies()
         dev = self.build_device
         half = torch.float16 if torch.device(dev).type == 'cuda' else None
 
@@ -264,7 +274,9 @@ class IndexStaged(nn.Module):
         add launches).  The query is rotated on the device
         (``kernels.rotate``); given the same rotated query the results are
         those of the host refine."""
-        if self.storage_full_cuda is None:
+        assert self.storage_cuda is not None, \
+            'call .to(device) first (again after a new build)'
+        if self.storage_full_cuda is None or self._full_prepared is None:
             self.stage_refine()
         device = self.cuda_device
         query = kernels.rotate(query.to(device).contiguous(), self.VT_cuda)

@@ -153,6 +153,30 @@ def test_repeated_rows_and_large_values(device):
     assert torch.allclose(d2[:300].cpu().double(), want, rtol=1e-5)
 
 
+def test_a_few_large_coordinates_do_not_spoil_the_table(device):
+    """A heavy-tailed column (a few coordinates thousands of times the rest):
+    the half-precision copy is scaled by the rows' typical length, not by the
+    largest coordinate, so the other coordinates keep their precision and the
+    table is still the exact one for the ordinary rows."""
+    n, d, k = 20000, 64, 10
+    g = torch.Generator().manual_seed(31)
+    x = torch.randn(n, d, generator=g)
+    wild = torch.arange(0, n, 97)
+    x[wild, 5] *= 5000.0
+    ids, d2 = utils.knn_graph(x.to(device), k)
+    tame = torch.ones(n, dtype=torch.bool)
+    tame[wild] = False
+    rows = torch.nonzero(tame).flatten()[:2000]
+    exact = torch.cdist(x[rows].double(), x.double()).square()
+    exact[torch.arange(rows.numel()), rows] = float('inf')
+    want = torch.topk(exact, k, dim=-1, largest=False)
+    got = ids[rows.to(device)].cpu()
+    hit = (got.unsqueeze(-1) == want.indices.unsqueeze(1)).any(1).float().mean()
+    print('heavy-tailed column: share of the exact table found', float(hit), flush=True)
+    assert float(hit) > 0.999
+    assert torch.allclose(d2[rows.to(device)].cpu().double(), want.values, rtol=1e-4)
+
+
 def test_knn_argument_errors(device):
     lib = _lib.lib()
     buf = torch.zeros(1 << 16, device=device)
@@ -251,6 +275,26 @@ def test_pruning_straight_from_the_rows(n, d, k, m_keep, fill, device):
     with pytest.raises(RuntimeError):
         kernels.graph_prune_rows(x, cand[:, :1].expand(-1, 300).contiguous(),
                                  cand_d[:, :1].expand(-1, 300).contiguous(), m_keep, fill)
+
+
+def test_pruning_drops_a_candidate_beyond_the_rows(device):
+    """A row number at or beyond the number of rows is no candidate: nothing
+    is read for it (it would lie outside the arrays) and the selection is that
+    of the same lists ending in -1 there."""
+    n, d, k = 3000, 64, 24
+    x = utils.gaussian_mixture(n, d, 8, 1.0, seed=77).to(device)
+    cand, cand_d = utils.knn_graph(x, k)
+    ended = cand.clone()
+    ended[::3, -4:] = -1
+    beyond = cand.clone()
+    beyond[::3, -4:] = torch.tensor([n, n + 1, 1 << 40, (1 << 62) + 5], device=device)
+    dist = cand_d.clone()
+    dist[::3, -4:] = float('inf')
+    want = kernels.graph_prune_rows(x, ended, dist, 12, True)
+    got = kernels.graph_prune_rows(x, beyond, dist, 12, True)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    assert int(got[::3].max()) < k - 4
 
 
 def test_pruning_of_more_nodes_than_one_launch_takes(device):

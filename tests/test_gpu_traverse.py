@@ -53,6 +53,14 @@ CASES = [
     (3000, 64, 40, 24, 'nsw', None, 24, 16, False),
     (5000, 64, 64, 64, 'nsw', 0.5, 128, 64, False),
     (5000, 32, 32, 32, 'nsw', 0.5, 512, 32, False),
+    # the instantiations the benchmark times, on graphs large enough for the
+    # lists to fill: the headline configuration's (128-float rows, 64
+    # neighbours, 64 entries, ef 32: traverse_kernel<128, 16>) and those of
+    # the 96-dimensional one (64-float rows, 32 neighbours, 32 entries, ef 64
+    # and 128: <256, 8> and <512, 8>)
+    (24000, 128, 128, 64, 'nsw', 0.25, 32, 64, False),
+    (24000, 96, 64, 32, 'nsw', 0.25, 64, 32, False),
+    (24000, 96, 64, 32, 'nsw', 0.25, 128, 32, False),
 ]
 
 
