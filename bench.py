@@ -246,24 +246,30 @@ class Stage:
         EP_I, EP_D = self.index.entry.search(self.query_cuda)
         return EP_I.contiguous(), EP_D.contiguous()
 
-    def traverse(self, ef, EP_I, EP_D, counters=None):
+    def traverse(self, ef, EP_I, EP_D, counters=None, wide=0):
+        """`wide` = 0: the exact mode; 1..4: the wide mode of that width."""
         out_I, out_D = self.buffers(ef)
-        self.kernels.traverse_prepared(
-            out_I, out_D, self.graph, self.index.storage_cuda,
-            self.query_cuda, EP_I, EP_D, counters)
+        if wide:
+            self.kernels.traverse_wide_prepared(
+                out_I, out_D, self.graph, self.index.storage_cuda,
+                self.query_cuda, EP_I, EP_D, counters, wide)
+        else:
+            self.kernels.traverse_prepared(
+                out_I, out_D, self.graph, self.index.storage_cuda,
+                self.query_cuda, EP_I, EP_D, counters)
         return out_I, out_D
 
-    def step(self, ef):
+    def step(self, ef, wide=0):
         EP_I, EP_D = self.entries()
-        return self.traverse(ef, EP_I, EP_D)
+        return self.traverse(ef, EP_I, EP_D, wide=wide)
 
 
-def end_to_end_recall(index, stage, ef, target, k):
+def end_to_end_recall(index, stage, ef, target, k, wide=0):
     """Recall of the whole three-stage search at this ef: device candidates,
     then the host refine on the full-dimension vectors.  Without a full
     graph (stage-only index): the recall of the candidate lists themselves."""
     from pilotann_amd import kernels, utils
-    out_I, out_D = stage.step(ef)
+    out_I, out_D = stage.step(ef, wide)
     torch.cuda.synchronize()
     buf_I = out_I.flatten(1).cpu()
     buf_D = out_D.flatten(1).cpu()
@@ -318,20 +324,20 @@ def measured_traffic(key, sources=TRAVERSAL_SOURCES):
             entry.get('kernel_sources_sha16') == kernel_sources_sha16(sources))
 
 
-def time_stage(stage, ef, steps, warmup):
+def time_stage(stage, ef, steps, warmup, wide=0):
     """Work counters of one launch (untimed), then `steps` timed passes of
     router + traversal; the traversal alone is bracketed by events on the
     launch stream."""
     device = stage.device
     EP_I, EP_D = stage.entries()
     counters = torch.zeros(5, dtype=torch.long, device=device)
-    out_I, out_D = stage.traverse(ef, EP_I, EP_D, counters)
+    out_I, out_D = stage.traverse(ef, EP_I, EP_D, counters, wide)
     torch.cuda.synchronize()
     counts = counters.cpu().tolist()
     launch_bytes = algorithmic_bytes(counts, stage.B, stage.index.d_principle,
                                      EP_I.size(1))
     for _ in range(warmup):
-        stage.step(ef)
+        stage.step(ef, wide)
     torch.cuda.synchronize()
     ev = [(torch.cuda.Event(enable_timing=True),
            torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
@@ -339,7 +345,7 @@ def time_stage(stage, ef, steps, warmup):
     for a, b in ev:
         EP_I, EP_D = stage.entries()
         a.record()
-        stage.traverse(ef, EP_I, EP_D)
+        stage.traverse(ef, EP_I, EP_D, wide=wide)
         b.record()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
@@ -815,8 +821,38 @@ def context_figures(line, args, cfg, index, stage, query, target, ef,
                              torch.equal(outs[1][1], out_D))}
     del outs
 
+    line['config']['wide_mode'] = wide_mode_figures(
+        cfg, index, stage, target, ef, args, line['config']['recall_at_k'])
+
     if args.power_law_twin:
         line['config']['power_law_spectrum'] = spectrum_twin(cfg, device, args)
+
+
+def wide_mode_figures(cfg, index, stage, target, ef, args, exact_recall):
+    """The labelled throughput mode (`pa_traverse_wide`: several nodes
+    expanded per step, result and open list one sorted pool) on the same
+    step: rate, algorithmic bytes of its own work over its kernel time, and
+    the recall of the whole search with its candidates beside the exact
+    mode's.  Context: never `value`."""
+    out = {'what': 'pa_traverse_wide, width 4: not the host search step for '
+                   'step; distances of returned ids exact',
+           'ef': ef}
+    rec, _ = end_to_end_recall(index, stage, ef, target, cfg['k'], wide=4)
+    t = time_stage(stage, ef, max(3, args.steps // 2), 1, wide=4)
+    out.update(
+        recall_at_k=round(rec, 4), exact_mode_recall_at_k=exact_recall,
+        recall_delta=round(rec - exact_recall, 4),
+        queries_per_s=round(stage.B / (t['ms_per_step'] * 1e-3), 1),
+        ms_per_step=round(t['ms_per_step'], 4),
+        kernel_ms=round(t['kernel_ms'], 4),
+        algorithmic_bytes_per_launch=t['launch_bytes'],
+        achieved_GBps=round(t['achieved'], 1),
+        frac=round(t['achieved'] / HBM_PEAK_GBS, 4),
+        counters=dict(zip(['expanded', 'adjacency_entries', 'distances',
+                           'admitted', 'result_slots'], t['counts'])))
+    log(f'[bench] wide mode ef={ef}: {t["kernel_ms"]:.3f} ms, recall {rec:.4f} '
+        f'(exact {exact_recall:.4f}), frac {out["frac"]}')
+    return out
 
 
 def knn_figures(cfg, args, device):

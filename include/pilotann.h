@@ -164,6 +164,35 @@ int pa_traverse_static(int64_t *out_I, float *out_D, const int32_t *adj,
                        int dp, int n_init, int beam, int ef, int n_neighbors,
                        uint64_t *counters, void *stream);
 
+/*
+ * The wide mode of the traversal: a labelled throughput mode beside
+ * pa_traverse, never the default.  No counterpart in the reference's host
+ * search, which pa_traverse reproduces; its shape is that of the reference's
+ * device kernel (extension/traverse_cuda.cu:116-226: several nodes expanded
+ * per step, one shared visited set).  The result list and the open list are
+ * one pool of the best candidates seen (as many as pa_traverse's result list,
+ * rounded up to a multiple of 64), sorted by distance; a step expands the
+ * `width` (1..4) best candidates not yet expanded together and merges their
+ * fresh neighbours into the pool with a bitonic network; the search ends when
+ * every candidate in the pool is expanded, or after min(1024, 2 * beam * ef)
+ * expansions.  Same arguments, output layout, distance arithmetic and visited
+ * set as pa_traverse: the distance returned for an id is bit for bit the host
+ * search's.  The ids are those of a best-first search that expands in groups
+ * and keeps its open list as long as its result list; they are not promised
+ * to equal traverse_cpu's (the recall of the whole search is the measure).
+ * Ids must fit 30 bits.  workspace: pa_traverse_wide_plan()'s bytes.
+ */
+int pa_traverse_wide_plan(int64_t n_storage, int64_t batch, int dp,
+                          int ef_total, int *n_slots, size_t *workspace_bytes);
+int pa_traverse_wide(int64_t *out_I, float *out_D, const int32_t *adj,
+                     const int32_t *gid, const int64_t *mapping,
+                     const float *storage, const float *query,
+                     const int64_t *init_I, const float *init_D, int64_t batch,
+                     int64_t n_nodes, int64_t n_storage, int dp, int n_init,
+                     int beam, int ef, int n_neighbors, int width,
+                     void *workspace, size_t workspace_bytes,
+                     uint64_t *counters, void *stream);
+
 /* ---- entry router -------------------------------------------------------- */
 
 /*

@@ -27,6 +27,11 @@ _SIGNATURES = {
     'pa_traverse_static': (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
                                   _i64, _i64, _i64, _int, _int, _int, _int,
                                   _int, _vp, _vp]),
+    'pa_traverse_wide_plan': (_int, [_i64, _i64, _int, _int,
+                                     ctypes.POINTER(_int), ctypes.POINTER(_sz)]),
+    'pa_traverse_wide': (_int, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
+                                _i64, _i64, _i64, _int, _int, _int, _int, _int,
+                                _int, _vp, _sz, _vp, _vp]),
     'pa_route': (_int, [_vp, _vp, _vp, _vp, _vp, _i64, _int, _int, _int,
                         _vp, _vp, _vp]),
     'pa_rotate': (_int, [_vp, _vp, _vp, _i64, _int, _int, _vp]),

@@ -10,7 +10,7 @@ ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, 'csrc')
 LIB = os.path.join(CSRC, 'libpilotann.so')
 
-HIP_SOURCES = ['traverse.hip', 'refine.hip', 'route.hip', 'rotate.hip',
+HIP_SOURCES = ['traverse.hip', 'traverse_wide.hip', 'refine.hip', 'route.hip', 'rotate.hip',
                'knn.hip', 'pipeline.hip']
 CXX_SOURCES = ['host_search.cpp']
 

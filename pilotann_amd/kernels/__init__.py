@@ -135,7 +135,8 @@ def traverse_cuda(output_I: torch.Tensor,
                   initial_I: torch.Tensor,
                   initial_D: torch.Tensor,
                   n_neighbors: int,
-                  counters: torch.Tensor = None):
+                  counters: torch.Tensor = None,
+                  mode: str = 'exact', width: int = 4):
     """Same arguments as ``kernels.traverse_cuda``
     (``pilot_ann/kernels/__init__.py:62-75``; checks of
     ``traverse_cuda.cu:256-281``).  ``output_*`` are ``[B, 4, ef]``; row b,
@@ -143,6 +144,8 @@ def traverse_cuda(output_I: torch.Tensor,
     (``traverse_cpu.cpp:12-163`` with ``ef_search = k = 4·ef``) best first,
     ``-1`` / ``+inf`` in unused slots.  ``n_neighbors`` may be any value up
     to 64.  ``counters`` (5 int64 on the device) is an optional work tally.
+    ``mode='wide'`` runs the labelled throughput mode instead
+    (:func:`traverse_wide_prepared`): not the host search step for step.
     """
     _check(indptr, 'indptr', 1, torch.int64, True)
     _check(indices, 'indices', 1, torch.int64, True)
@@ -175,7 +178,13 @@ def traverse_cuda(output_I: torch.Tensor,
         _check(counters, 'counters', 1, torch.int64, True)
         _require(counters.numel() >= 5, 'counters.numel() >= 5')
 
+    _require(mode in ('exact', 'wide'), "mode in ('exact', 'wide')")
     graph = prepare_graph(indptr, indices, mapping, n_storage, n_neighbors)
+    if mode == 'wide':
+        _require(1 <= width <= 4, '1 <= width <= 4')
+        traverse_wide_prepared(output_I, output_D, graph, storage, query,
+                               initial_I, initial_D, counters, width)
+        return
     traverse_prepared(output_I, output_D, graph, storage, query, initial_I,
                       initial_D, counters)
 
@@ -202,6 +211,35 @@ def traverse_prepared(output_I, output_D, graph: PreparedGraph, storage,
             _ptr(initial_D), batch_size, graph.n_nodes, graph.n_storage,
             d_model, initial_I.size(-1), beam, ef_search, graph.n_neighbors,
             _ptr(ws), ws.numel(), _ptr(counters), _stream()), 'pa_traverse')
+
+
+def traverse_wide_prepared(output_I, output_D, graph: PreparedGraph, storage,
+                           query, initial_I, initial_D, counters=None,
+                           width: int = 4):
+    """The wide mode of the traversal (``pa_traverse_wide``), a labelled
+    throughput mode beside :func:`traverse_prepared`, never the default: same
+    arguments and output layout, the ``width`` (1..4) best open candidates
+    expanded together per step, result list and open list one sorted pool.
+    Distances of returned ids are the exact mode's, bit for bit; the ids are
+    not promised to be the host search's (``traverse_cpu``)."""
+    lib = _lib.lib()
+    storage = prepare_rows(storage).rows
+    batch_size, d_model = query.shape
+    ef_search = output_I.size(-1)
+    beam = output_I.size(1)
+    with torch.cuda.device(query.device):
+        nbytes = ctypes.c_size_t()
+        _lib.check(lib.pa_traverse_wide_plan(
+            graph.n_storage, batch_size, d_model, beam * ef_search, None,
+            ctypes.byref(nbytes)), 'pa_traverse_wide_plan')
+        ws = _workspace(query.device, nbytes.value)
+        _lib.check(lib.pa_traverse_wide(
+            _ptr(output_I), _ptr(output_D), _ptr(graph.adj), _ptr(graph.gid),
+            _ptr(graph.mapping), _ptr(storage), _ptr(query), _ptr(initial_I),
+            _ptr(initial_D), batch_size, graph.n_nodes, graph.n_storage,
+            d_model, initial_I.size(-1), beam, ef_search, graph.n_neighbors,
+            int(width), _ptr(ws), ws.numel(), _ptr(counters), _stream()),
+            'pa_traverse_wide')
 
 
 # ---- entry router -----------------------------------------------------------
