@@ -135,5 +135,28 @@ def route(query, route_vectors, entry_vectors):
     return router, dist
 
 
+def traverse_wide(output_I, output_D, initial_I, initial_D, indptr, indices,
+                  mapping, storage, query, width=4, counters=None):
+    """The library's wide mode (``pa_traverse_wide``) restated: ``storage``
+    rows by global id like :func:`traverse_cpu`, ``mapping`` global id →
+    storage row (orders exact distance ties as the device does), outputs
+    ``[B, k]`` written in place."""
+    batch, d_model = query.shape
+    assert storage.shape[1] == d_model and mapping.shape[0] == storage.shape[0]
+    assert output_I.shape == output_D.shape and output_I.shape[0] == batch
+    assert initial_I.shape == initial_D.shape and initial_I.shape[0] == batch
+    cptr = None
+    if counters is not None:
+        assert counters.size >= N_COUNTERS
+        cptr = _i64(counters)
+    rc = lib().orc_traverse_wide(
+        _i64(output_I), _f32(output_D), _i64(initial_I), _f32(initial_D),
+        _i64(indptr), _i64(indices), _i64(mapping), _f32(storage), _f32(query),
+        ctypes.c_int64(batch), ctypes.c_int64(storage.shape[0]), d_model,
+        initial_I.shape[1], output_I.shape[1], int(width), cptr)
+    if rc:
+        raise RuntimeError(f'oracle traverse_wide: error {rc}')
+
+
 def num_threads() -> int:
     return lib().orc_num_threads()

@@ -14,6 +14,9 @@
  *   batch driver (one stage) ... extension/traverse_cpu.cpp:167-257
  *   batch driver (refine) ...... extension/traverse_cpu.cpp:261-369
  *   leaf distances of the router extension/routing_cuda.cu:10-66
+ * and, with no counterpart in the reference, the library's own wide mode
+ * (orc_traverse_wide, at the end): restated here so that the device kernel of
+ * that mode has a checker too; what pins it is stated there.
  *
  * Floating point: the reference accumulates (q-x)^2 with one FMA per element
  * into eight independent lanes (element j goes to lane j mod 8) and then adds
@@ -417,6 +420,182 @@ int orc_route(int64_t *router, float *dist, const float *query,
             dist[b * n_leaves + l] =
                 orc_square_dist(q, leaves + l * (int64_t)d, d, 0);
     }
+    return 0;
+}
+
+/* ---- the wide mode of the device traversal ---------------------------------
+ *
+ * Not a restatement of anything in the reference: the library's labelled
+ * throughput mode (pa_traverse_wide), written down once more in plain C so
+ * that the device kernel can be compared id for id.  A best-first search
+ * whose result list and open list are one pool of the P best candidates seen
+ * (P = the heap size of the ladder for k, rounded up to a multiple of 64),
+ * ordered by (distance, storage row):
+ *   - the entries are marked and offered to the pool, 64 at a time (one
+ *     without a storage row keeps its global id and is never expanded);
+ *   - a step takes the `width` first candidates of the pool that are not yet
+ *     expanded, walks their rows of neighbours in that order (a row ends at
+ *     its first negative id; nodes without a storage row are skipped), marks
+ *     what is new and offers it, with its distance, to the pool, 64 at a
+ *     time in that order: of a group of 64 those strictly below the pool's
+ *     last key enter, the pool keeps its P smallest;
+ *   - the search ends when no candidate of the pool is left to expand, or
+ *     after min(1024, 2k) expansions.
+ * Pins: the distances are orc_square_dist's; with width 1 and a pool that
+ * holds every node the result is the exact nearest neighbours on a connected
+ * graph (brute force, tests/test_oracle_wide.py); the stop rule, the cap and
+ * the order of a step are stepped by hand there on small graphs.
+ */
+#define ORC_WIDE_DONE 0x80000000u
+#define ORC_WIDE_GLOBAL 0x40000000u
+#define ORC_WIDE_ID 0x3fffffffu
+
+typedef struct {
+    int32_t key;   /* order-preserving integer image of the float distance */
+    uint32_t val;  /* storage row, or DONE | GLOBAL | global id */
+} orc_wide_entry;
+
+static int32_t orc_float_key(float x) {
+    int32_t b;
+    memcpy(&b, &x, 4);
+    return b ^ ((b >> 31) & 0x7fffffff);
+}
+
+static float orc_key_float(int32_t k) {
+    int32_t b = k ^ ((k >> 31) & 0x7fffffff);
+    float x;
+    memcpy(&x, &b, 4);
+    return x;
+}
+
+static int orc_wide_less(const orc_wide_entry *a, const orc_wide_entry *b) {
+    if (a->key != b->key) return a->key < b->key;
+    return a->val < b->val;
+}
+
+static int orc_wide_cmp(const void *a, const void *b) {
+    const orc_wide_entry *x = a, *y = b;
+    return orc_wide_less(x, y) ? -1 : orc_wide_less(y, x) ? 1 : 0;
+}
+
+/* offers `n` staged entries to the pool, 64 at a time */
+static void orc_wide_offer(orc_wide_entry *pool, int P, orc_wide_entry *staged,
+                           int n, orc_wide_entry *tmp, int64_t *admitted) {
+    for (int base = 0; base < n; base += 64) {
+        const int32_t worst = pool[P - 1].key;
+        int m = 0;
+        memcpy(tmp, pool, (size_t)P * sizeof(*pool));
+        for (int i = base; i < n && i < base + 64; ++i)
+            if (staged[i].key < worst) tmp[P + m++] = staged[i];
+        if (!m) continue;
+        if (admitted) *admitted += m;
+        qsort(tmp, (size_t)(P + m), sizeof(*tmp), orc_wide_cmp);
+        memcpy(pool, tmp, (size_t)P * sizeof(*pool));
+    }
+}
+
+int orc_traverse_wide(int64_t *out_I, float *out_D, const int64_t *init_I,
+                      const float *init_D, const int64_t *indptr,
+                      const int64_t *indices, const int64_t *mapping,
+                      const float *storage, const float *query, int64_t batch,
+                      int64_t n_nodes, int d, int n_init, int k, int width,
+                      int64_t *counters) {
+    const int H = orc_heap_size(k);
+    if (H < 0 || d % ORC_LANES || width < 1 || width > 4) return -1;
+    const int P = (H + 63) / 64 * 64;
+    const int max_iter = 2 * k < 1024 ? 2 * k : 1024;
+    int64_t n_rows = 0;
+    for (int64_t g = 0; g < n_nodes; ++g)
+        if (mapping[g] >= n_rows) n_rows = mapping[g] + 1;
+    int64_t *gid = malloc((size_t)(n_rows ? n_rows : 1) * sizeof(*gid));
+    for (int64_t g = 0; g < n_nodes; ++g)
+        if (mapping[g] >= 0) gid[mapping[g]] = g;
+    int64_t total[ORC_N_COUNTERS] = {0, 0, 0, 0, 0};
+#pragma omp parallel
+    {
+        unsigned char *seen = malloc((size_t)(n_rows ? n_rows : 1));
+        orc_wide_entry *pool = malloc((size_t)(P + 64) * sizeof(*pool));
+        orc_wide_entry *tmp = malloc((size_t)(P + 64) * sizeof(*tmp));
+        orc_wide_entry *staged = malloc(4 * 64 * sizeof(*staged));
+        int64_t mine[ORC_N_COUNTERS] = {0, 0, 0, 0, 0};
+#pragma omp for schedule(guided)
+        for (int64_t b = 0; b < batch; ++b) {
+            const float *q = query + b * d;
+            memset(seen, 0, (size_t)n_rows);
+            for (int i = 0; i < P; ++i) {
+                pool[i].key = 0x7f800000;
+                pool[i].val = 0xffffffffu;
+            }
+            /* the entries */
+            for (int base = 0; base < n_init; base += 64) {
+                int n = 0;
+                for (int i = base; i < n_init && i < base + 64; ++i) {
+                    const int64_t g = init_I[b * n_init + i];
+                    if (g < 0 || g >= n_nodes) continue;
+                    staged[n].key = orc_float_key(init_D[b * n_init + i]);
+                    if (mapping[g] >= 0) {
+                        seen[mapping[g]] = 1;
+                        staged[n].val = (uint32_t)mapping[g];
+                    } else {
+                        staged[n].val = ORC_WIDE_DONE | ORC_WIDE_GLOBAL | (uint32_t)g;
+                    }
+                    ++n;
+                }
+                orc_wide_offer(pool, P, staged, n, tmp, NULL);
+            }
+            int n_expand = 0;
+            while (n_expand < max_iter) {
+                int want = width < max_iter - n_expand ? width : max_iter - n_expand;
+                int64_t chosen[4];
+                int n_chosen = 0;
+                for (int i = 0; i < P && n_chosen < want; ++i)
+                    if (!(pool[i].val & ORC_WIDE_DONE)) {
+                        chosen[n_chosen++] = pool[i].val & ORC_WIDE_ID;
+                        pool[i].val |= ORC_WIDE_DONE;
+                    }
+                if (!n_chosen) break;
+                n_expand += n_chosen;
+                int n = 0;
+                for (int w = 0; w < n_chosen; ++w) {
+                    const int64_t u = gid[chosen[w]];
+                    for (int64_t e = indptr[u]; e < indptr[u + 1]; ++e) {
+                        const int64_t v = indices[e];
+                        if (v < 0) break;
+                        mine[1] += 1;
+                        const int64_t row = v < n_nodes ? mapping[v] : -1;
+                        if (row < 0 || seen[row]) continue;
+                        seen[row] = 1;
+                        staged[n].key = orc_float_key(
+                            orc_square_dist(q, storage + v * d, d, 0));
+                        staged[n].val = (uint32_t)row;
+                        ++n;
+                    }
+                }
+                mine[2] += n;
+                orc_wide_offer(pool, P, staged, n, tmp, &mine[3]);
+            }
+            mine[0] += n_expand;
+            mine[4] += k;
+            for (int i = 0; i < k; ++i) {
+                const uint32_t val = pool[i].val;
+                int64_t id = -1;
+                if (val != 0xffffffffu)
+                    id = (val & ORC_WIDE_GLOBAL) ? (int64_t)(val & ORC_WIDE_ID)
+                                                 : gid[val & ORC_WIDE_ID];
+                out_I[b * k + i] = id;
+                out_D[b * k + i] = orc_key_float(pool[i].key);
+            }
+        }
+#pragma omp critical
+        for (int c = 0; c < ORC_N_COUNTERS; ++c) total[c] += mine[c];
+        free(seen);
+        free(pool);
+        free(tmp);
+        free(staged);
+    }
+    if (counters)
+        for (int c = 0; c < ORC_N_COUNTERS; ++c) counters[c] += total[c];
+    free(gid);
     return 0;
 }
 

@@ -203,15 +203,19 @@ class IndexStaged(nn.Module):
     @torch.no_grad()
     def search(self, query: torch.Tensor, k: int, ef_search: int,
                chunk_size: int = 128, refine: str = 'host',
-               rotate: str = 'device'):
+               rotate: str = 'device', traversal: str = 'exact'):
         """``rotate='device'`` (default on a GPU) uploads the query and
         rotates it there (``kernels.rotate``), then copies the rotated query
         back for the host refine; ``rotate='host'`` is the reference's host
-        matmul (``layers/staged.py:198``).  The two agree to float rounding."""
+        matmul (``layers/staged.py:198``).  The two agree to float rounding.
+        ``traversal='wide'`` (with ``refine='device'``) takes the candidates
+        from the labelled throughput mode of the traversal
+        (``kernels.traverse_wide_prepared``) instead of the exact one."""
         assert query.dim() == 2
+        assert traversal in ('exact', 'wide')
         if refine == 'device':
-            return self._search_on_device(query, k, ef_search)
-        assert refine == 'host'
+            return self._search_on_device(query, k, ef_search, traversal)
+        assert refine == 'host' and traversal == 'exact'
         if rotate == 'device' and self.VT_cuda is not None:
             rotated = kernels.rotate(
                 query.to(device=self.cuda_device).contiguous(), self.VT_cuda)
@@ -265,7 +269,7 @@ class IndexStaged(nn.Module):
                              max(ef_search, k))
         return topk_I, topk_D
 
-    def _search_on_device(self, query, k, ef_search):
+    def _search_on_device(self, query, k, ef_search, traversal='exact'):
         """All three stages on the device: entries, subgraph traversal, refine,
         top-k copied back at the end.  A batch of 2048 queries or more is
         searched as two halves on two streams: while the last searches of one
@@ -295,10 +299,12 @@ class IndexStaged(nn.Module):
             self.mapping_cuda, self.storage_cuda.size(0), self.n_neighbors)
         full = self._full_prepared
 
+        traverse = (kernels.traverse_wide_prepared if traversal == 'wide'
+                    else kernels.traverse_prepared)
+
         def run(lo, hi):
-            kernels.traverse_prepared(
-                cand_I[lo:hi], cand_D[lo:hi], sub, self.storage_cuda,
-                query_cuda[lo:hi], EP_I[lo:hi], EP_D[lo:hi])
+            traverse(cand_I[lo:hi], cand_D[lo:hi], sub, self.storage_cuda,
+                     query_cuda[lo:hi], EP_I[lo:hi], EP_D[lo:hi])
             c_I, c_D = cand_I[lo:hi].flatten(1), cand_D[lo:hi].flatten(1)
             kernels.traverse_refine_cuda(
                 topk_I[lo:hi], topk_D[lo:hi], c_I, c_D, c_I, c_D, sub, full,

@@ -110,6 +110,13 @@ def test_index_staged_end_to_end(device):
     # a query that is already on the device: same rotation, same answer
     gpu_I, gpu_D = index.search(q.to(device), k=k, ef_search=32, refine='device')
     assert torch.equal(gpu_I, dev_I) and torch.equal(gpu_D, dev_D)
+    # candidates from the wide mode of the traversal: a search of the same
+    # quality (its ids are not promised to be the exact mode's)
+    wide_I, wide_D = index.search(q, k=k, ef_search=32, refine='device',
+                                  traversal='wide')
+    assert abs(utils.recall(wide_I, target) - utils.recall(dev_I, target)) <= 0.002
+    ref = torch.cdist(q.unsqueeze(1), x[wide_I]).squeeze(1).square()
+    assert torch.allclose(wide_D, ref, atol=1e-3)
     # the reference's host matmul instead: another summation order, results
     # of the same quality
     host_I, host_D = index.search(q, k=k, ef_search=32, chunk_size=128,

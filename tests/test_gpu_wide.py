@@ -78,6 +78,16 @@ def test_wide_mode_properties(case, device):
         ids, counts = np.unique(I[b][real], return_counts=True)
         twice = set(ids[counts > 1].tolist())
         assert twice <= set(init_I[b].tolist())
+    # id for id the search the oracle restates (ties aside)
+    k = 4 * ef
+    I_ref = np.empty((I.shape[0], k), np.int64)
+    D_ref = np.empty((I.shape[0], k), np.float32)
+    ref = np.zeros(5, np.int64)
+    oracle.traverse_wide(I_ref, D_ref, init_I.numpy().copy(), init_D.numpy().copy(),
+                         p.sub_indptr.numpy(), p.sub_indices.numpy(),
+                         p.mapping.numpy(), xr, qr, width, ref)
+    assert_same_search(I, D, I_ref, D_ref)
+    assert cnt[0] == ref[0] and cnt[2] == ref[2] and cnt[3] == ref[3]
     # the candidates are as good as the exact mode's
     I_exact, D_exact, _ = run(p, dp, ef, init_I, init_D, device, 'exact')
     r_wide, r_exact = reduced_recall(p, dp, I), reduced_recall(p, dp, I_exact)
