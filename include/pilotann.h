@@ -144,12 +144,14 @@ int pa_traverse(int64_t *out_I, float *out_D, const int32_t *adj,
  * PA_STATIC_SCRATCH_BYTES inside the library (each GPU the library runs on
  * holds one until the process ends), and the call allocates nothing.
  *
- * A resident wavefront needs ceil(n_storage / 32) words rounded up to 1 KiB
- * plus 4 bytes per cell of its result list; as many wavefronts are launched as
- * the array holds (fewer than pa_traverse would use when the index is large,
- * which costs time, not correctness).  PA_E_STATIC when fewer than
- * min(batch, 256) fit: with the largest lists that is n_storage above about
- * 4.1 million rows.
+ * A resident wavefront needs its visited slice (ceil(n_storage / 32) words
+ * rounded up to 1 KiB), 8 bytes per entry of its log of admitted candidates
+ * (2 H + 128 entries, H = pa_heap_size(beam * ef)) and, with the longest
+ * lists only (H = 2048), 16.6 KB for the last two levels of its open list; as
+ * many wavefronts are launched as the array holds (fewer than pa_traverse
+ * would use when the index is large, which costs time, not correctness).
+ * PA_E_STATIC when fewer than min(batch, 256) fit: with the longest lists
+ * that is n_storage above about 3.7 million rows (4.1 million at H = 512).
  *
  * All calls on one GPU share the array: calls that may overlap on one GPU
  * (different streams, different threads) race; serialise them.  Nothing is

@@ -52,8 +52,11 @@ def both_entry_points(p, dp, ef, n_init, seed, device):
 def test_static_scratch_entry_point_equals_pa_traverse(device):
     big = Problem(n=9000, d=64, deg=48, sample_ratio=0.5, seed=61, n_query=700)
     small = Problem(n=2500, d=32, deg=16, sample_ratio=0.25, seed=62, n_query=37)
+    # the third call with the longest lists (ef 512: 4096 cells, whose last
+    # two levels live in the array as well)
     for name, p, dp, ef, n_init in (('first call', big, 64, 96, 48),
-                                    ('second, smaller call', small, 32, 8, 8)):
+                                    ('second, smaller call', small, 32, 8, 8),
+                                    ('third call, longest lists', small, 32, 512, 8)):
         print('static scratch:', name, flush=True)
         (I_a, D_a, c_a), (I_b, D_b, c_b) = both_entry_points(p, dp, ef, n_init, 3, device)
         assert (I_a != -7).all() and (I_b != -7).all()
