@@ -650,7 +650,8 @@ def main():
     recall_at = [s for s in sweep if s['ef'] == ef][0]['recall']
 
     t = time_stage(stage, ef, args.steps, args.warmup)
-    out_I, out_D = t['out_I'], t['out_D']
+    # copies: later measurements (other ef, the wide mode) reuse the buffers
+    out_I, out_D = t['out_I'].clone(), t['out_D'].clone()
     launch_bytes, ms_per_step = t['launch_bytes'], t['ms_per_step']
     key = traffic_key(cfg, B, ef)
 

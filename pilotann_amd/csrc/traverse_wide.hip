@@ -43,7 +43,10 @@ using namespace pa;
 
 namespace {
 
-constexpr int kMaxWidth = 4;
+#ifndef PA_WIDE_MAX_WIDTH
+#define PA_WIDE_MAX_WIDTH 4
+#endif
+constexpr int kMaxWidth = PA_WIDE_MAX_WIDTH;
 constexpr unsigned kDone = 0x80000000u;     // expanded, or nothing to expand
 constexpr unsigned kGlobal = 0x40000000u;   // the low bits are a global id, not a storage row
 constexpr unsigned kIdMask = 0x3fffffffu;
@@ -450,7 +453,7 @@ int make_wide_plan(int64_t n_storage, int64_t batch, int dp, int ef_total, WideP
     }
     if (per_cu < 1) per_cu = 1;
 #ifndef PA_WIDE_MAX_WAVES_PER_CU
-#define PA_WIDE_MAX_WAVES_PER_CU 16
+#define PA_WIDE_MAX_WAVES_PER_CU 20
 #endif
     if (per_cu > PA_WIDE_MAX_WAVES_PER_CU) per_cu = PA_WIDE_MAX_WAVES_PER_CU;
     int64_t slots = (int64_t)per_cu * cus;
