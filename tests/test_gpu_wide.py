@@ -116,3 +116,60 @@ def test_wide_mode_argument_errors(device):
         torch.empty(0, 8, dtype=torch.long, device=device),
         torch.empty(0, 8, device=device), 32, mode='wide')
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize('seed', range(60))
+def test_wide_mode_on_random_graphs(seed, device):
+    """The random graphs of the exact mode's sweep (every pool size, vector
+    lengths with and without a specialised kernel, degrees 1..64, ragged
+    rows, self loops, repeated and unsampled neighbours and entries, exact
+    ties), widths 1..4, against the CPU restatement."""
+    from test_gpu_fuzz import make_case
+    c = make_case(5000 + seed)
+    width = 1 + seed % 4
+    print('wide fuzz', {k: c[k] for k in ('seed', 'n_nodes', 'n_rows', 'deg', 'dp', 'ef',
+                                          'n_init', 'B', 'tied', 'unsampled_neighbours')},
+          'width', width, flush=True)
+    B, k = c['B'], 4 * c['ef']
+    xn, qn = c['x'].numpy(), c['query'].numpy()
+    init_D = np.stack([oracle.square_dist(qn[b].copy(), xn, c['init_I'][b].numpy().copy())
+                       for b in range(B)])
+    ref_I = np.empty((B, k), np.int64)
+    ref_D = np.empty((B, k), np.float32)
+    ref = np.zeros(5, np.int64)
+    oracle.traverse_wide(ref_I, ref_D, c['init_I'].numpy().copy(), init_D.copy(),
+                         c['indptr'].numpy(), c['indices'].numpy(), c['mapping'].numpy(),
+                         xn, qn, width, ref)
+    out_I = torch.empty(B, 4, c['ef'], dtype=torch.long, device=device)
+    out_D = torch.empty(B, 4, c['ef'], dtype=torch.float, device=device)
+    cnt = torch.zeros(5, dtype=torch.long, device=device)
+    kernels.traverse_cuda(
+        output_I=out_I, output_D=out_D, indptr=c['indptr'].to(device),
+        indices=c['indices'].to(device), mapping=c['mapping'].to(device),
+        storage=c['x'][c['nodelist']].contiguous().to(device),
+        query=c['query'].to(device), initial_I=c['init_I'].to(device),
+        initial_D=torch.from_numpy(init_D).to(device), n_neighbors=c['deg'],
+        counters=cnt, mode='wide', width=width)
+    torch.cuda.synchronize()
+    got_I = out_I.flatten(1).cpu().numpy()
+    got_D = out_D.flatten(1).cpu().numpy()
+    if not c['tied']:
+        assert_same_search(got_I, got_D, ref_I, ref_D)
+        cnt = cnt.cpu().numpy()
+        assert cnt[2] == ref[2] and cnt[3] == ref[3]
+        # An entry named twice sits in the pool twice, and its second copy is
+        # expanded too, to no effect; whether that copy is still in the pool
+        # when its turn comes can depend on the order inside the tie (the two
+        # are equal but for the flag).  Expansions agree up to those copies.
+        repeats = sum(len(row) - len(set(row)) for row in c['init_I'].tolist())
+        assert abs(int(cnt[0]) - int(ref[0])) <= repeats
+        return
+    # exact ties: which of several equally distant candidates is expanded or
+    # kept first may differ (the order inside a tie is by storage row, and the
+    # flag of an expanded entry takes part in it); every id must still carry
+    # its own exact distance, best first
+    for b in range(B):
+        real = got_I[b] >= 0
+        assert (got_D[b][1:] >= got_D[b][:-1]).all()
+        assert np.array_equal(got_D[b][real],
+                              oracle.square_dist(qn[b].copy(), xn, got_I[b][real].copy()))
