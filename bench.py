@@ -80,6 +80,7 @@ def log(*a):
 
 
 TRAVERSAL_SOURCES = ('traverse.hip', 'search_lists.h', 'device_common.h')
+WIDE_SOURCES = ('traverse_wide.hip', 'search_lists.h', 'device_common.h')
 
 
 def kernel_sources_sha16(names=TRAVERSAL_SOURCES):
@@ -505,14 +506,15 @@ def cpu_full_graph_baseline(index, query, stage, target, k, budget_s=6.0):
                 cores=oracle.num_threads(), passes=passes, sweep=sweep)
 
 
-def stage_record(t, B, key):
-    traffic, fresh = measured_traffic(key)
+def stage_record(t, B, key, kernel='traverse_kernel'):
+    traffic, fresh = measured_traffic(key + ('/wide' if kernel == 'wide_kernel' else ''),
+                                      WIDE_SOURCES if kernel == 'wide_kernel' else TRAVERSAL_SOURCES)
     rec = {
         'bound': 'hbm', 'achieved': round(t['achieved'], 1),
         'peak': HBM_PEAK_GBS, 'unit': 'GB/s',
         'frac': round(t['achieved'] / HBM_PEAK_GBS, 4),
         'traffic': traffic,
-        'kernel': 'traverse_kernel',
+        'kernel': kernel,
         'kernel_ms': round(t['kernel_ms'], 4),
         'algorithmic_bytes_per_launch': t['launch_bytes'],
         'counters': dict(zip(['expanded', 'adjacency_entries', 'distances',
@@ -565,6 +567,11 @@ def main():
                     help="only time the graph builder's nearest-neighbour "
                          "kernel (pa_knn) on the configuration's base set "
                          "against itself, print its rate and exit")
+    ap.add_argument('--traversal', default='exact', choices=['exact', 'wide'],
+                    help="'wide': sweep and time the labelled throughput mode "
+                         "(pa_traverse_wide) instead of the exact traversal; the "
+                         "line says so in config.traversal (for profiles of that "
+                         "kernel; the default run reports it as config.wide_mode)")
     ap.add_argument('--power-law-twin', action='store_true',
                     help='also build the configuration on data with a '
                          'power-law spectrum (exponent 0.5) and measure recall '
@@ -634,8 +641,9 @@ def main():
     efs = [args.ef] if args.ef else cfg['ef_sweep']
     if args.curve and not args.ef:
         efs = cfg.get('curve', efs)
+    wide = 4 if args.traversal == 'wide' else 0
     for ef in efs:
-        rec, refine_s = end_to_end_recall(index, stage, ef, target, k)
+        rec, refine_s = end_to_end_recall(index, stage, ef, target, k, wide)
         sweep.append(dict(ef=ef, recall=round(rec, 4),
                           refine_qps=round(B / refine_s, 1)
                           if refine_s == refine_s else None))
@@ -649,7 +657,7 @@ def main():
     ef = chosen
     recall_at = [s for s in sweep if s['ef'] == ef][0]['recall']
 
-    t = time_stage(stage, ef, args.steps, args.warmup)
+    t = time_stage(stage, ef, args.steps, args.warmup, wide)
     # copies: later measurements (other ef, the wide mode) reuse the buffers
     out_I, out_D = t['out_I'].clone(), t['out_D'].clone()
     launch_bytes, ms_per_step = t['launch_bytes'], t['ms_per_step']
@@ -679,10 +687,13 @@ def main():
                           'graph, no refine)' if index.fullgraph is None else
                           'whole search: device candidates, then host refine'),
             'stage': 'routing_cuda + traverse_cuda (GPU search stage)',
+            'traversal': ('exact: traverse_cpu step for step' if not wide else
+                          'wide: the labelled throughput mode, not the host '
+                          'search step for step (not the headline figure)'),
             # data, ground truth and the index on the device, when built here
             'index_build_seconds': cfg.get('index_build_seconds'),
         },
-        'roofline': stage_record(t, B, key),
+        'roofline': stage_record(t, B, key, 'wide_kernel' if wide else 'traverse_kernel'),
     }
     others = [e for e in (efs if args.curve else
                           ALSO_TIMED.get(args.config, []))
@@ -692,19 +703,20 @@ def main():
         line['config']['other_ef'] = []
         for e in others:
             if e not in recalls:
-                recalls[e] = round(end_to_end_recall(index, stage, e, target, k)[0], 4)
-            o = time_stage(stage, e, max(3, args.steps // 2), 1)
-            rec = stage_record(o, B, traffic_key(cfg, B, e))
+                recalls[e] = round(end_to_end_recall(index, stage, e, target, k, wide)[0], 4)
+            o = time_stage(stage, e, max(3, args.steps // 2), 1, wide)
+            rec = stage_record(o, B, traffic_key(cfg, B, e),
+                               'wide_kernel' if wide else 'traverse_kernel')
             line['config']['other_ef'].append(dict(
                 ef=e, recall_at_k=recalls[e],
                 queries_per_s=round(B / (o['ms_per_step'] * 1e-3), 1),
                 ms_per_step=round(o['ms_per_step'], 4), roofline=rec))
             log(f'[bench] ef={e}: {o["kernel_ms"]:.3f} ms, frac {rec["frac"]}')
-    if not args.no_context:
+    if not args.no_context and not wide:
         context_figures(line, args, cfg, index, stage, query, target, ef,
                         launch_bytes, out_D)
 
-    if not args.no_cpu_baseline:
+    if not args.no_cpu_baseline and not wide:
         EP_I, EP_D = stage.entries()
         torch.cuda.synchronize()
         base, (ref_I, ref_D) = cpu_baseline(index, stage, ef, EP_I, EP_D)
@@ -851,6 +863,10 @@ def wide_mode_figures(cfg, index, stage, target, ef, args, exact_recall):
         frac=round(t['achieved'] / HBM_PEAK_GBS, 4),
         counters=dict(zip(['expanded', 'adjacency_entries', 'distances',
                            'admitted', 'result_slots'], t['counts'])))
+    traffic, fresh = measured_traffic(traffic_key(cfg, stage.B, ef) + '/wide',
+                                      WIDE_SOURCES)
+    if traffic is not None:
+        out.update(traffic=traffic, traffic_kernel_sources_unchanged=bool(fresh))
     log(f'[bench] wide mode ef={ef}: {t["kernel_ms"]:.3f} ms, recall {rec:.4f} '
         f'(exact {exact_recall:.4f}), frac {out["frac"]}')
     return out
