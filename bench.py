@@ -109,13 +109,18 @@ def make_data(cfg, device):
     return x, q, target
 
 
+def cache_key(cfg):
+    """What of a configuration decides the content of a stage cache."""
+    return {k: v for k, v in cfg.items() if k not in ('name', 'index_build_seconds')}
+
+
 def save_stage_cache(path, cfg, index, q, target):
     """What the device stage of a `stage_only` configuration needs, so that a
     counter run does not pay for the index build again: rotation, sample,
     subgraph, router, queries, ground truth and the sampled rows' first
     d_principle coordinates."""
     torch.save({
-        'config': {k: v for k, v in cfg.items() if k != 'name'},
+        'config': cache_key(cfg),
         'VT': index.VT, 'nodelist': index.nodelist, 'mapping': index.mapping,
         'subgraph.indptr': index.subgraph.indptr,
         'subgraph.indices': index.subgraph.indices,
@@ -129,7 +134,7 @@ def load_stage_cache(path, cfg, device):
     from pilotann_amd import IndexStaged
     from pilotann_amd.layers.staged import GraphModule
     saved = torch.load(path, weights_only=True)
-    if saved['config'] != {k: v for k, v in cfg.items() if k != 'name'}:
+    if saved['config'] != cache_key(cfg):
         raise SystemExit(f'{path} was written for another configuration')
     index = IndexStaged(d_model=cfg['d'], d_principle=cfg['dp'],
                         sample_ratio=cfg['ratio'], graph_method=cfg['graph'],
@@ -526,6 +531,39 @@ def stage_record(t, B, key, kernel='traverse_kernel'):
     return rec
 
 
+PHASES = ['pop', 'adjacency_and_visited_marks_issued', 'visited_marks_waited_for',
+          'rows_and_distances', 'inserts', 'per_query_set_up', 'per_query_results']
+
+
+def phase_split(stage, ef):
+    """Cycles per phase of the searches of one launch, from the tuning build
+    whose kernel reads the cycle counter at every phase boundary after waiting
+    for what the phase has outstanding: a phase's figure includes its memory
+    waits, and that build overlaps less than the shipped one (its duration is
+    reported beside the split, to compare)."""
+    EP_I, EP_D = stage.entries()
+    for _ in range(3):
+        counters = torch.zeros(12, dtype=torch.long, device=stage.device)
+        torch.cuda.synchronize()
+        started = time.perf_counter()
+        stage.traverse(ef, EP_I, EP_D, counters)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - started
+    c = counters.cpu().tolist()
+    cycles = c[5:12]
+    total = max(sum(cycles), 1)
+    return {
+        'phase_split': 'traverse_kernel built with -DPA_PHASE_TIMERS',
+        'ef': ef, 'queries': stage.B,
+        'launch_ms_of_the_timed_build': round(elapsed * 1e3, 3),
+        'expansions': c[0], 'distances': c[2], 'admitted': c[3],
+        'share_of_wavefront_cycles': {n: round(v / total, 4)
+                                      for n, v in zip(PHASES, cycles)},
+        'cycles_per_expansion': {n: round(v / max(c[0], 1), 1)
+                                 for n, v in zip(PHASES, cycles)},
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument('--gpus', type=int, default=1)
@@ -577,6 +615,12 @@ def main():
                          'power-law spectrum (exponent 0.5) and measure recall '
                          'and rate over a range of ef there (a second index '
                          'build; context, not part of `value`)')
+    ap.add_argument('--phase-split', action='store_true',
+                    help='only report where the searches of one launch spend '
+                         'their cycles (pop, adjacency and visited marks, rows, '
+                         'inserts, ...), measured with the tuning build of '
+                         '`python -m pilotann_amd.build --phase-timers` (needs '
+                         '--ef), and exit')
     ap.add_argument('--copy-calibration', action='store_true',
                     help='only run a plain 1 GiB device copy five times (to '
                          'scale the FETCH_SIZE / WRITE_SIZE counters) and exit')
@@ -606,6 +650,15 @@ def main():
                                      args, 'cuda:0')), flush=True)
         return
 
+    if args.phase_split:
+        from pilotann_amd import _lib, build
+        if not args.ef:
+            ap.error('--phase-split needs --ef')
+        if not os.path.exists(build.PHASE_LIB):
+            ap.error(f'{build.PHASE_LIB} not found: '
+                     'python -m pilotann_amd.build --phase-timers')
+        _lib.LIB_PATH = build.PHASE_LIB      # before the first library call
+
     cfg = dict(CONFIGS[args.config], name=args.config)
     if args.n_base:
         cfg['n'] = args.n_base
@@ -626,6 +679,10 @@ def main():
     index, query, target = build_index(cfg, device, args.stage_cache)
     stage = Stage(index, query, device)
     B, k, dp = stage.B, cfg['k'], cfg['dp']
+
+    if args.phase_split:
+        print(json.dumps(phase_split(stage, args.ef)), flush=True)
+        return
 
     if args.device_refine_only:
         if not args.ef:

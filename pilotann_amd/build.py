@@ -9,6 +9,10 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, 'csrc')
 LIB = os.path.join(CSRC, 'libpilotann.so')
+# tuning build whose traversal kernel tallies cycles per phase of a search
+# (``python -m pilotann_amd.build --phase-timers``; ``bench.py --phase-split``
+# loads it); not built by default and never the library the package loads
+PHASE_LIB = os.path.join(CSRC, 'libpilotann_phase_timers.so')
 
 HIP_SOURCES = ['traverse.hip', 'traverse_wide.hip', 'refine.hip', 'route.hip', 'rotate.hip',
                'knn.hip', 'pipeline.hip']
@@ -40,7 +44,7 @@ def build(verbose: bool = False, output: str = LIB,
           extra_hip_flags=()) -> str:
     """Compile everything and link ``output`` (default: the library the
     loader uses).  ``extra_hip_flags`` are added to the device compiles, e.g.
-    ``-DPA_PHASE_TIMERS`` for a tuning build written elsewhere."""
+    ``-DPA_PHASE_TIMERS`` for the tuning build ``PHASE_LIB``."""
     include = os.path.join(ROOT, 'include')
     objects = []
     for name in HIP_SOURCES:
@@ -66,4 +70,8 @@ def build(verbose: bool = False, output: str = LIB,
 
 
 if __name__ == '__main__':
-    print(build(verbose='-q' not in sys.argv))
+    if '--phase-timers' in sys.argv:
+        print(build(verbose='-q' not in sys.argv, output=PHASE_LIB,
+                    extra_hip_flags=['-DPA_PHASE_TIMERS']))
+    else:
+        print(build(verbose='-q' not in sys.argv))

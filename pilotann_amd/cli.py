@@ -51,7 +51,7 @@ class Profiler:
 
     def __init__(self, dataset, algorithm, n_queries, d_principle,
                  entry_method, sample_ratio, device, refine='host',
-                 data_root='.dataset', seed=7):
+                 data_root='.dataset', seed=7, traversal='exact'):
         self.algorithm = algorithm
         self.n_queries = n_queries
         self.d_principle = d_principle
@@ -59,6 +59,7 @@ class Profiler:
         self.sample_ratio = sample_ratio
         self.device = device
         self.refine = refine
+        self.traversal = traversal
         self.seed = seed
         self.index = None
         self.method = None
@@ -124,7 +125,8 @@ class Profiler:
     def search_pilot(self, query, k, ef_search):
         before = time.perf_counter()
         out = self.index.search(query, k=k, ef_search=ef_search,
-                                chunk_size=CHUNK_SIZE, refine=self.refine)[0].cpu()
+                                chunk_size=CHUNK_SIZE, refine=self.refine,
+                                traversal=self.traversal)[0].cpu()
         return out, time.perf_counter() - before
 
     def search_host(self, query, k, ef_search):
@@ -164,6 +166,10 @@ def main(argv=None):
                         help="directory of the reference's dataset folders")
     parser.add_argument('--refine', choices=['host', 'device'], default='host',
                         help="where stages 2 and 3 run (the reference: host)")
+    parser.add_argument('--traversal', choices=['exact', 'wide'], default='exact',
+                        help="'wide': the labelled throughput mode of the "
+                        "device stage (several nodes per step; other candidates "
+                        "than the host kernel's, --refine device only)")
     parser.add_argument('--methods', type=lambda s: s.split(','),
                         default=['search-pilot', 'host-cpu'])
     parser.add_argument('--n_repeats', type=int, default=20)
@@ -174,13 +180,15 @@ def main(argv=None):
     args = parser.parse_args(argv)
     if not torch.cuda.is_available():
         raise SystemExit('pilotann_amd.cli: no GPU')
+    if args.traversal == 'wide' and args.refine != 'device':
+        raise SystemExit('pilotann_amd.cli: --traversal wide needs --refine device')
 
     profiler = Profiler(dataset=args.dataset, algorithm=args.algorithm,
                         entry_method=args.router,
                         sample_ratio=args.sample_ratio,
                         d_principle=args.d_principle, n_queries=args.n_queries,
                         device=args.device, refine=args.refine,
-                        data_root=args.data_root)
+                        data_root=args.data_root, traversal=args.traversal)
     if args.load:
         profiler.load(args.load)
     records = {method: [] for method in args.methods}

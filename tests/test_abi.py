@@ -44,6 +44,15 @@ def test_host_only_entry_points():
                                4, 100, 60, 8, 10, 16) == -3
     assert lib.pa_pipeline(*([None] * 15), 100, 1000, 250, 64, 32, 32, 32, 16,
                            10, 30, None) == -9
+    # the wide mode: width 1..4, ids of 30 bits, then the pointers
+    wide = [None] * 9
+    assert lib.pa_traverse_wide(*wide, 4, 1000, 500, 64, 8, 4, 8, 16, 5, None, 0,
+                                None, None) == -2
+    assert lib.pa_traverse_wide(*wide, 4, (1 << 30) + 1, 500, 64, 8, 4, 8, 16, 4,
+                                None, 0, None, None) == -10
+    assert lib.pa_traverse_wide(*wide, 4, 1000, 500, 60, 8, 4, 8, 16, 4, None, 0,
+                                None, None) == -3
+    assert lib.pa_traverse_wide_plan(500, 4, 64, 4096, None, None) == -5
     assert lib.pa_rotate(None, None, None, 4, 60, 8, None) == -3
     assert lib.pa_rotate(None, None, None, 4, 64, 65, None) == -2
     assert lib.pa_rotate(None, None, None, 4, 64, 8, None) == -1

@@ -152,6 +152,16 @@ def test_command_line_benchmark_prints_the_reference_lines(device, capsys):
     assert [r['ef_search'] for r in records['search-pilot']] == [16, 32]
     # more effort, better recall
     assert records['search-pilot'][1]['recall'] >= records['search-pilot'][0]['recall']
+    # the labelled wide traversal: device refine only, recall within a point
+    wide = cli.main(['--dataset', 'synth:20000x64:16:0.5', '--d_principle', '32',
+                     '--n_neighbors', '32', '--router', 'router16x32',
+                     '--ef_search', '32', '--n_queries', '256', '--n_repeats', '3',
+                     '--refine', 'device', '--traversal', 'wide',
+                     '--methods', 'search-pilot', '--device', str(device)])
+    assert abs(wide['search-pilot'][0]['recall']
+               - records['search-pilot'][1]['recall']) < 0.02
+    with pytest.raises(SystemExit):
+        cli.main(['--traversal', 'wide', '--device', str(device)])
 
 
 def test_command_line_benchmark_reads_the_reference_dataset_layout(device, capsys, tmp_path):
