@@ -56,9 +56,16 @@ class Problem:
         return ids.contiguous(), torch.from_numpy(dist)
 
 
-def assert_same_search(I_a, D_a, I_b, D_b):
+def assert_same_search(I_a, D_a, I_b, D_b, worst_tie=None):
     """Distances identical bit for bit; ids identical except inside a run of
-    equal distances of one row, where only the set has to agree."""
+    equal distances of one row, where only the set has to agree.
+
+    ``worst_tie(row, ids)`` (optional) is asked when the sets differ at the
+    worst distance a row keeps: two candidates at exactly that distance
+    competed for the last place, and which of them a list drops first is
+    heap-structure detail with no effect on the search.  It gets the ids of
+    the first list at that distance and must check that each is a candidate
+    at exactly that distance."""
     D_a, D_b = np.asarray(D_a), np.asarray(D_b)
     I_a, I_b = np.asarray(I_a), np.asarray(I_b)
     assert D_a.shape == D_b.shape and I_a.shape == I_b.shape
@@ -68,7 +75,13 @@ def assert_same_search(I_a, D_a, I_b, D_b):
         f'{np.argwhere(~same_d)[0]}')
     bad = np.argwhere((I_a != I_b).any(-1)).flatten()
     for r in bad:
+        real = I_a[r] >= 0
+        worst = D_a[r][real].max() if real.any() else None
         for dist in np.unique(D_a[r][I_a[r] != I_b[r]]):
             sel = D_a[r] == dist
-            assert sorted(I_a[r][sel]) == sorted(I_b[r][sel]), (
+            if sorted(I_a[r][sel]) == sorted(I_b[r][sel]):
+                continue
+            assert worst_tie is not None and dist == worst, (
                 f'row {r}: ids differ outside a tie at distance {dist}')
+            assert (I_a[r][sel] >= 0).all() and (I_b[r][sel] >= 0).all()
+            worst_tie(int(r), I_a[r][sel], dist)

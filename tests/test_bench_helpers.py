@@ -54,3 +54,29 @@ def test_traffic_figures_name_the_sources_they_were_measured_with():
     assert bench.measured_traffic('no such workload') == (None, None)
     cfg = dict(bench.CONFIGS['c3'], name='c3')
     assert bench.traffic_key(cfg, 10000, 32) in entries
+
+
+def test_the_parity_check_of_the_gpu_tests_tolerates_ties_only():
+    """tests/common.py:assert_same_search — what the GPU parity tests pass or
+    fail on: another order inside a tie passes, another id does not, another
+    member of a tie passes only at the worst kept distance and only through
+    the caller's check of those ids."""
+    import pytest
+    from common import assert_same_search
+    D = np.array([[1.0, 2.0, 2.0, 3.0, 3.0]], np.float32)
+    I = np.array([[5, 6, 7, 8, 9]])
+    swapped = np.array([[5, 7, 6, 9, 8]])
+    assert_same_search(I, D, swapped, D.copy())
+    other = np.array([[5, 6, 7, 8, 4]])
+    with pytest.raises(AssertionError, match='outside a tie'):
+        assert_same_search(other, D, I, D.copy())
+    asked = []
+    assert_same_search(other, D, I, D.copy(),
+                       worst_tie=lambda row, ids, dist: asked.append((row, sorted(ids), dist)))
+    assert asked == [(0, [4, 8], 3.0)]
+    # not at the worst distance: never tolerated
+    inner = np.array([[5, 6, 4, 8, 9]])
+    with pytest.raises(AssertionError, match='outside a tie'):
+        assert_same_search(inner, D, I, D.copy(), worst_tie=lambda *a: None)
+    with pytest.raises(AssertionError, match='distances differ'):
+        assert_same_search(I, D, I, D + 1)

@@ -108,7 +108,12 @@ def test_random_graph(seed, device):
     got_I = out_I.flatten(1).cpu().numpy()
     got_D = out_D.flatten(1).cpu().numpy()
     if not c['tied']:
-        assert_same_search(got_I, got_D, ref_I, ref_D)
+        # random rows tie by chance now and then; at the worst kept distance
+        # the two lists may then keep different members of the tie
+        def at_that_distance(b, ids, dist):
+            assert np.array_equal(oracle.square_dist(qn[b].copy(), xn, ids.copy()),
+                                  np.full(len(ids), dist, np.float32))
+        assert_same_search(got_I, got_D, ref_I, ref_D, worst_tie=at_that_distance)
         return
     # With exact ties among the kept distances the two result lists may keep
     # different members of a tie (which of several equally bad entries leaves

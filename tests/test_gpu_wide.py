@@ -154,7 +154,11 @@ def test_wide_mode_on_random_graphs(seed, device):
     got_I = out_I.flatten(1).cpu().numpy()
     got_D = out_D.flatten(1).cpu().numpy()
     if not c['tied']:
-        assert_same_search(got_I, got_D, ref_I, ref_D)
+        # a chance tie at the worst kept distance may keep another member
+        def at_that_distance(b, ids, dist):
+            assert np.array_equal(oracle.square_dist(qn[b].copy(), xn, ids.copy()),
+                                  np.full(len(ids), dist, np.float32))
+        assert_same_search(got_I, got_D, ref_I, ref_D, worst_tie=at_that_distance)
         cnt = cnt.cpu().numpy()
         assert cnt[2] == ref[2] and cnt[3] == ref[3]
         # An entry named twice sits in the pool twice, and its second copy is
