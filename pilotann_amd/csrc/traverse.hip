@@ -119,11 +119,22 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
     // constant that fits the instruction's offset field.
     using Open = OpenList<H, deep_from(H)>;
     constexpr int S = (H + kWave - 1) / kWave;
-    constexpr int kSortN = H <= kWave ? kWave : 1 << (floor_log2(H - 1) + 1);
+    // cells of the final sort: all of them, and those sorted in LDS at once
+    constexpr int kSortAll = H <= kWave ? kWave : 1 << (floor_log2(H - 1) + 1);
+    constexpr int kSortLds = kSortAll > 1024 ? 1024 : kSortAll;
     constexpr int kHeapCells =
-        Open::kLdsCells > kSortN ? Open::kLdsCells : kSortN;
+        Open::kLdsCells > kSortLds ? Open::kLdsCells : kSortLds;
+    // The table of recently marked rows in front of the bitmask: half the
+    // size for the long lists, whose residency is bound by LDS (lists of 2048
+    // and 4096 cells: 9 instead of 8 wavefronts per compute unit, 5 % faster
+    // on 10 000 queries over 500 000 rows of 128 floats although the table
+    // answers fewer tests; a quarter of the size is slower again, and
+    // where LDS does not bound the residency the smaller table only costs).
+    constexpr int kSeenLog2 =
+        H >= 1024 && kSeenCacheLog2 > 0 ? kSeenCacheLog2 - 1 : kSeenCacheLog2;
+    constexpr int kSeen = 1 << kSeenLog2;
     struct Lds {
-        uint32_t seen_cache[kSeenCache];
+        uint32_t seen_cache[kSeen];
         int cand_id[kWave];
         float cand_key[kWave];
         float query[DP8 ? query_floats(8 * DP8) : 4];
@@ -141,7 +152,7 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
     float *qv = DP8 ? lds.query : query_any_length;
     const int dp = DP8 ? DP8 * 8 : a.dp;
     uint32_t *seen_cache = lds.seen_cache;
-    const bool use_cache = a.n_storage <= (0xffff << kSeenCacheLog2);
+    const bool use_cache = a.n_storage <= (0xffff << kSeenLog2);
     const int deg = a.deg;
     uint32_t *seen = a.seen + (size_t)blockIdx.x * (size_t)a.slot_stride;
     // after the visited slice: the log of admitted candidates, then the
@@ -172,7 +183,7 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
                 *reinterpret_cast<uint4 *>(seen + w) = make_uint4(0, 0, 0, 0);
         for (int i = lane; i < dp; i += kWave)
             qv[query_slot(i, dp >> 3)] = a.query[(size_t)q * dp + i];
-        for (int i = lane; i < kSeenCache; i += kWave) seen_cache[i] = 0xffffffffu;
+        for (int i = lane; i < kSeen; i += kWave) seen_cache[i] = 0xffffffffu;
         open.reset(lane);
         ResultKeys<S> res;
         res.init(H, lane);
@@ -242,8 +253,8 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
         auto test_and_set = [&](int v) -> uint32_t {
             uint32_t before = 0xffffffffu;
             if (v >= 0) {
-                const int cell = v & (kSeenCache - 1);
-                const uint32_t tag = (uint32_t)v >> kSeenCacheLog2;
+                const int cell = v & (kSeen - 1);
+                const uint32_t tag = (uint32_t)v >> kSeenLog2;
                 const uint32_t ways = use_cache ? seen_cache[cell] : 0xffffffffu;
                 if (!use_cache || ((ways & 0xffffu) != tag && (ways >> 16) != tag)) {
                     before = atomicOr(&seen[v >> 5], 1u << (v & 31));
@@ -354,15 +365,40 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
         // maximum as many as make H — into the LDS the open list no longer
         // needs, padded to a power of two with +inf, and sorted there.
         wave_sync();
-        for (int i = lane; i < a.sort_n; i += kWave)
-            okey[i] = INFINITY, oval[i] = -1;
         ResultLog::settle();
         int n_below = 0;
         for (int base = 0; base < log.n; base += kWave) {
             const int i = base + lane;
             n_below += __popcll(__ballot(i < log.n && log.entry[i].x < res.worst));
         }
-        {
+        // Stages of a bitonic network over okey / oval [0, n): merges of
+        // `first_size` cells and up (2: a full sort; n: the last merge alone,
+        // for cells that are bitonic already); `desc`: largest first.
+        auto lds_sort = [&](int n, int first_size, bool desc) {
+            for (int size = first_size; size <= n; size <<= 1) {
+                for (int stride = size >> 1; stride > 0; stride >>= 1) {
+                    for (int t = lane; t < (n >> 1); t += kWave) {
+                        const int i = ((t & ~(stride - 1)) << 1) | (t & (stride - 1));
+                        const int j = i | stride;
+                        const float ki = okey[i], kj = okey[j];
+                        const int vi = oval[i], vj = oval[j];
+                        const bool gt = ki > kj || (ki == kj && vi > vj);
+                        const bool lt = ki < kj || (ki == kj && vi < vj);
+                        if ((((i & size) == 0) != desc) ? gt : lt) {
+                            okey[i] = kj, oval[i] = vj;
+                            okey[j] = ki, oval[j] = vi;
+                        }
+                    }
+                    wave_sync();
+                }
+            }
+        };
+        int64_t *oI = a.out_I + (size_t)q * a.k;
+        float *oD = a.out_D + (size_t)q * a.k;
+        if constexpr (kSortAll <= kSortLds) {
+            for (int i = lane; i < a.sort_n; i += kWave)
+                okey[i] = INFINITY, oval[i] = -1;
+            wave_sync();
             int at_below = 0, at_worst = n_below;
             for (int base = 0; base < log.n; base += kWave) {
                 const int i = base + lane;
@@ -381,30 +417,83 @@ __global__ __launch_bounds__(kWave) PA_OCCUPANCY(H) void traverse_kernel(Travers
                 at_below += __popcll(mb);
                 at_worst += __popcll(mt);
             }
-        }
-        wave_sync();
-        for (int size = 2; size <= a.sort_n; size <<= 1) {
-            for (int stride = size >> 1; stride > 0; stride >>= 1) {
-                for (int t = lane; t < (a.sort_n >> 1); t += kWave) {
-                    const int i = ((t & ~(stride - 1)) << 1) | (t & (stride - 1));
-                    const int j = i | stride;
-                    const float ki = okey[i], kj = okey[j];
-                    const int vi = oval[i], vj = oval[j];
-                    const bool gt = ki > kj || (ki == kj && vi > vj);
-                    const bool lt = ki < kj || (ki == kj && vi < vj);
-                    if ((i & size) == 0 ? gt : lt) {
-                        okey[i] = kj, oval[i] = vj;
-                        okey[j] = ki, oval[j] = vi;
+            wave_sync();
+            lds_sort(a.sort_n, 2, false);
+            for (int i = lane; i < a.k; i += kWave) {
+                oI[i] = (int64_t)oval[i];
+                oD[i] = okey[i];
+            }
+        } else {
+            // The longest lists sort in two halves of kSortLds cells, so that
+            // the sort does not decide the size of the LDS block (and with it
+            // how many wavefronts a compute unit holds).  The set is
+            // compacted at the head of the log (in log order: a write lands
+            // on an entry already read), as (distance, id); the first half is
+            // sorted ascending and the second descending through LDS; one
+            // exchange between the halves in the log leaves every cell of the
+            // first below every cell of the second and both bitonic; each is
+            // then merged in LDS and written out.
+            static_assert(kSortAll == 2 * kSortLds, "two halves");
+            static_assert(ResultLog::capacity_for(H) >= kSortAll, "the log holds them");
+            int m = 0, ties_left = H - n_below;
+            for (int base = 0; base < log.n; base += kWave) {
+                const int i = base + lane;
+                int2 e = make_int2(0x7fffffff, -1);
+                if (i < log.n) e = log.entry[i];
+                const bool below = i < log.n && e.x < res.worst;
+                const bool tie = i < log.n && e.x == res.worst;
+                const unsigned long long mt = __ballot(tie);
+                const bool keep = below || (tie && lane_rank(mt) < ties_left);
+                const unsigned long long mk = __ballot(keep);
+                if (keep) {
+                    const int id = e.y < -1 ? -2 - e.y : a.gid[e.y];
+                    log.entry[m + lane_rank(mk)] =
+                        make_int2(__float_as_int(key_to_float(e.x)), id);
+                }
+                m += __popcll(mk);
+                ties_left -= min(ties_left, (int)__popcll(mt));
+            }
+            ResultLog::settle();
+            auto load_half = [&](int half) {
+                for (int i = lane; i < kSortLds; i += kWave) {
+                    const int at = half * kSortLds + i;
+                    int2 e = make_int2(__float_as_int(INFINITY), -1);
+                    if (at < m) e = log.entry[at];
+                    okey[i] = __int_as_float(e.x), oval[i] = e.y;
+                }
+                wave_sync();
+            };
+            for (int half = 0; half < 2; ++half) {
+                load_half(half);
+                lds_sort(kSortLds, 2, half == 1);
+                for (int i = lane; i < kSortLds; i += kWave)
+                    log.entry[half * kSortLds + i] =
+                        make_int2(__float_as_int(okey[i]), oval[i]);
+                wave_sync();
+            }
+            ResultLog::settle();
+            m = kSortAll;  // both halves are whole now, +inf cells included
+            for (int i = lane; i < kSortLds; i += kWave) {
+                const int2 x = log.entry[i], y = log.entry[kSortLds + i];
+                const float kx = __int_as_float(x.x), ky = __int_as_float(y.x);
+                if (kx > ky || (kx == ky && x.y > y.y)) {
+                    log.entry[i] = y;
+                    log.entry[kSortLds + i] = x;
+                }
+            }
+            ResultLog::settle();
+            for (int half = 0; half < 2; ++half) {
+                load_half(half);
+                lds_sort(kSortLds, kSortLds, false);
+                for (int i = lane; i < kSortLds; i += kWave) {
+                    const int r = half * kSortLds + i;
+                    if (r < a.k) {
+                        oI[r] = (int64_t)oval[i];
+                        oD[r] = okey[i];
                     }
                 }
                 wave_sync();
             }
-        }
-        int64_t *oI = a.out_I + (size_t)q * a.k;
-        float *oD = a.out_D + (size_t)q * a.k;
-        for (int i = lane; i < a.k; i += kWave) {
-            oI[i] = (int64_t)oval[i];
-            oD[i] = okey[i];
         }
         wave_sync();
 
