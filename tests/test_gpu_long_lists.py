@@ -111,3 +111,34 @@ def test_refine_top_100_matches_oracle(index, device):
     assert_same_search(init_I.cpu().numpy(), init_D.cpu().numpy(),
                        ref_init_I, ref_init_D)
     assert_same_search(out_I.cpu().numpy(), out_D.cpu().numpy(), ref_I, ref_D)
+
+
+def test_longest_lists_when_wavefronts_take_a_second_query(index, device):
+    """More queries than a launch has wavefronts (9 per compute unit with the
+    lists of 4096 cells), so that a wavefront starts a query on the log whose
+    head the last query's two-part sort has rewritten: the 48 queries 60 times
+    over, every copy equal to the oracle's answer for its query."""
+    ef, reps = 512, 60
+    k = 4 * ef
+    ref_I = np.empty((B, k), np.int64)
+    ref_D = np.empty((B, k), np.float32)
+    oracle.traverse_cpu(ref_I, ref_D, index.init_I.numpy().copy(),
+                        index.init_D.numpy().copy(), index.sub_indptr.numpy(),
+                        index.sub_indices.numpy(), index.xr, index.qr, k)
+    n = B * reps
+    out_I = torch.empty(n, 4, ef, dtype=torch.long, device=device)
+    out_D = torch.empty(n, 4, ef, dtype=torch.float, device=device)
+    storage = torch.from_numpy(index.xr)[index.nodelist].contiguous().to(device)
+    kernels.traverse_cuda(
+        out_I, out_D, index.sub_indptr.to(device), index.sub_indices.to(device),
+        index.mapping.to(device), storage,
+        torch.from_numpy(index.qr).to(device).repeat(reps, 1).contiguous(),
+        index.init_I.to(device).repeat(reps, 1).contiguous(),
+        index.init_D.to(device).repeat(reps, 1).contiguous(), DEG)
+    torch.cuda.synchronize()
+    got_I = out_I.flatten(1).cpu().numpy().reshape(reps, B, k)
+    got_D = out_D.flatten(1).cpu().numpy().reshape(reps, B, k)
+    assert_same_search(got_I[0], got_D[0], ref_I, ref_D)
+    for r in range(1, reps):
+        assert np.array_equal(got_D[r], got_D[0]), f'copy {r}: distances'
+        assert np.array_equal(got_I[r], got_I[0]), f'copy {r}: ids'
